@@ -1,0 +1,165 @@
+#!/usr/bin/env python3
+"""Headline benchmark: one rank's 8-partial reduce + residual + RMSNorm + per-token fp8 quant stage
+at 2048 x 8192 bf16 (BASELINE config c3) on ONE MI355X, through the C ABI (tde_reduce_rms).
+
+A step is one launch of the fused row kernel over one batch of synthetic inputs that already sit
+in HBM.  Inputs rotate over several distinct sets (> 1 GiB in total) so that no launch finds its
+inputs in the 256 MB Infinity Cache.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3] [--no-cpu-baseline]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
+
+BENCH_CONFIGS = {
+    # name: (N, T, H, dtype, sigma, eps, quant)
+    "c2": (8, 128, 4096, "bf16", 0.5, 1e-5, "none"),
+    "c3": (8, 2048, 8192, "bf16", 0.5, 1e-5, "fp8_token"),
+    "c4": (4, 8192, 7168, "bf16", 1.0, 1e-6, "fp8_group"),
+    "c5": (4, 32768, 5120, "f16", 1.0, 1e-6, "int8_token"),
+}
+
+
+def make_sets(torch, cfg, nsets, dev):
+    N, T, H, dt, sigma, eps, quant = cfg
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dt]
+    g = torch.Generator(device=dev).manual_seed(1234)
+    sets = []
+    for _ in range(nsets):
+        parts = [(torch.randn((T, H), generator=g, device=dev, dtype=torch.float32) * sigma).to(dtype) for _ in range(N)]
+        residual = torch.randn((T, H), generator=g, device=dev, dtype=torch.float32).to(dtype)
+        res_out = torch.empty_like(residual)
+        q = torch.empty((T, H), dtype=torch.uint8, device=dev) if quant != "none" else None
+        nscale = T * (H // 128) if quant == "fp8_group" else T
+        scale = torch.empty((nscale,), dtype=torch.float32, device=dev) if quant != "none" else None
+        norm = torch.empty_like(residual) if quant == "none" else None
+        sets.append(dict(parts=parts, residual=residual, res_out=res_out, q=q, scale=scale, norm=norm))
+    gamma = (torch.rand((H,), generator=g, device=dev, dtype=torch.float32) + 0.5).to(dtype)
+    return sets, gamma, dtype
+
+
+def cpu_baseline(torch, cfg, budget_s=15.0):
+    """The oracle's torch-eager composition timed on the host cores, on a bounded sample: as many
+    full-size passes of the same workload as fit in about budget_s (at least 2 after one warm-up)."""
+    from oracle import eager
+    N, T, H, dt, sigma, eps, quant = cfg
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dt]
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)
+    torch.set_num_threads(cores)
+    rows = min(T, 2048)
+    parts, residual, gamma = eager.make_inputs(N, rows, H, dtype, sigma, seed=3)
+    eager.reduce_rms(parts, residual, gamma, eps, quant)  # warm-up
+    times = []
+    t_begin = time.perf_counter()
+    while len(times) < 2 or (time.perf_counter() - t_begin < budget_s and len(times) < 50):
+        t0 = time.perf_counter()
+        eager.reduce_rms(parts, residual, gamma, eps, quant)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": rows / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": "%d passes of %d rows x %d (%s, N=%d, %s), median; torch-eager oracle on host CPU" % (
+            len(times), rows, H, dt, N, quant),
+        "ms_per_pass": med * 1e3,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="c3", choices=sorted(BENCH_CONFIGS))
+    ap.add_argument("--sets", type=int, default=0, help="distinct input sets to rotate over (0 = enough for > 1 GiB)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--algo", default="auto", choices=["auto", "fused", "staged"])
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (one rank's stage with N local partial buffers); "
+              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from torch_dist_ext_amd import _capi
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cfg = BENCH_CONFIGS[args.config]
+    N, T, H, dt, sigma, eps, quant = cfg
+    qm = {"none": _capi.QUANT_NONE, "fp8_token": _capi.QUANT_FP8_TOKEN, "fp8_group": _capi.QUANT_FP8_GROUP,
+          "int8_token": _capi.QUANT_INT8_TOKEN}[quant]
+    algo = {"auto": _capi.ALGO_AUTO, "fused": _capi.ALGO_FUSED, "staged": _capi.ALGO_STAGED}[args.algo]
+    dcode = {"bf16": _capi.BF16, "f16": _capi.F16, "f32": _capi.F32}[dt]
+    prob = _capi.make_problem(dcode, N, T, H, eps, quant=qm, algo=algo, write_norm=0)
+    plan = _capi.plan(prob)
+    bytes_per_launch = plan.algorithmic_bytes
+    nsets = args.sets or max(2, -(-(1 << 30) // bytes_per_launch) + 1)
+    sets, gamma, dtype = make_sets(torch, cfg, nsets, dev)
+    stage = torch.empty((T, H), dtype=dtype, device=dev) if algo == _capi.ALGO_STAGED else None
+    stream = torch.cuda.current_stream(dev)
+
+    def launch(s):
+        _capi.reduce_rms(prob, [p.data_ptr() for p in s["parts"]], s["residual"].data_ptr(), s["res_out"].data_ptr(),
+                         gamma.data_ptr(), norm_out=s["norm"].data_ptr() if s["norm"] is not None else None,
+                         q_out=s["q"].data_ptr() if s["q"] is not None else None,
+                         scale_out=s["scale"].data_ptr() if s["scale"] is not None else None,
+                         stage=stage.data_ptr() if stage is not None else None, stream=stream.cuda_stream)
+
+    for i in range(args.warmup):
+        launch(sets[i % nsets])
+    torch.cuda.synchronize(dev)
+
+    # Timed region: exactly K steps; HIP events on the launch stream bracket every launch.
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    torch.cuda.synchronize(dev)
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        starts[i].record(stream)
+        launch(sets[i % nsets])
+        ends[i].record(stream)
+    torch.cuda.synchronize(dev)
+    wall = time.perf_counter() - t0
+    per_launch_ms = sorted(s.elapsed_time(e) for s, e in zip(starts, ends))
+    avg_ms = sum(per_launch_ms) / len(per_launch_ms)
+    med_ms = per_launch_ms[len(per_launch_ms) // 2]
+    span_ms = starts[0].elapsed_time(ends[-1])
+
+    ms_per_step = wall * 1e3 / args.steps
+    gbs_job = bytes_per_launch / (wall / args.steps) / 1e9
+    achieved = bytes_per_launch / (avg_ms * 1e-3) / 1e9
+    out = {
+        "metric": "achieved HBM GB/s, one rank's 8-partial reduce+residual+RMSNorm+per-token fp8 stage",
+        "value": gbs_job, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dt, "data": "synthetic",
+        "tokens_per_s": T / (wall / args.steps),
+        "pct_of_hbm_peak": 100.0 * gbs_job / HBM_PEAK_GBS,
+        "config": {"workload": "%s: N=%d partials [%d,%d] %s, residual add + RMSNorm + %s" % (args.config, N, T, H, dt, quant),
+                   "algo": args.algo, "input_sets": nsets, "block_threads": plan.block_threads,
+                   "grid_blocks": plan.grid_blocks, "algorithmic_bytes": bytes_per_launch},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel_avg_us": avg_ms * 1e3, "kernel_median_us": med_ms * 1e3,
+                     "event_span_us_per_step": span_ms * 1e3 / args.steps},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch, cfg)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,167 @@
+/*
+ * tde_abi.h — C ABI of the MI355X (gfx950) fused reduce + residual + RMSNorm (+ dynamic quant)
+ * row kernels.  Plain pointers and sizes only: no torch types, no C++ types.
+ *
+ * The library behind this header (libtde_hip.so) computes ONE rank's reduce-and-normalize stage
+ * of the reference's fused `allreduce_rms` operator.  The N peer partial buffers that the
+ * reference reads through IPC-mapped peer memory are N ordinary device allocations here.
+ *
+ * Reference interfaces replaced (paths relative to the reference tree):
+ *   - allreduce_rms_fusion_impl<T>(void** workspace, rank, nranks, size, hidden_dim, in, res_in,
+ *     res_out, norm_out, gamma, eps, stream)       src/common/all_reduce_fusion_impl.h:500-535
+ *   - AllReduceFusionParams<T>                      src/common/all_reduce_fusion_impl.h:300-314
+ *   - allreduce_fusion_kernel_launcher<T,NRanks>    src/common/all_reduce_fusion_impl.h:476-498
+ *   - CommWorkspace allocation + pointer table      src/ops/all_reduce_fusion.cpp:63-105,143-174
+ *
+ * Every function returns a tde_status (0 = success).  HIP runtime failures are returned as
+ * TDE_EHIP; the HIP error code is then available from tde_last_hip_error().
+ */
+#ifndef TDE_ABI_H
+#define TDE_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TDE_ABI_VERSION 1
+#define TDE_MAX_RANKS 16 /* array bound, as MAX_RANKS in src/ops/all_reduce_fusion.h:8 */
+#define TDE_QUANT_GROUP 128
+
+/* ---- status codes ------------------------------------------------------------------------- */
+typedef enum tde_status {
+    TDE_OK = 0,
+    TDE_EINVAL = 1,     /* null pointer / malformed struct */
+    TDE_ENRANKS = 2,    /* nranks not in {2,4,8}; reference: assert(false) impl.h:526-534 */
+    TDE_EDTYPE = 3,     /* dtype not supported */
+    TDE_ESHAPE = 4,     /* hidden*elem not a multiple of 16 bytes, tokens<0, hidden<=0 (impl.h:479-480) */
+    TDE_EHIDDEN = 5,    /* hidden larger than the row kernel supports (reference: pkg assert, __init__.py:69) */
+    TDE_EALIGN = 6,     /* a buffer is not 16-byte aligned (vec_t alignment, impl.h:208) */
+    TDE_EQUANT = 7,     /* unknown quant mode, or group mode with hidden % 128 != 0 */
+    TDE_EALGO = 8,      /* unknown algorithm, or staged algorithm without a stage buffer */
+    TDE_EHIP = 9,       /* HIP runtime error; see tde_last_hip_error() */
+    TDE_ERANK = 10,     /* rank outside [0,nranks) */
+    TDE_ENOMEM = 11     /* device allocation failed */
+} tde_status;
+
+/* ---- enums ---------------------------------------------------------------------------------- */
+typedef enum tde_dtype {
+    TDE_BF16 = 0, /* __bfloat16 in the reference dispatch, src/ops/all_reduce_fusion.cpp:19-22 */
+    TDE_F16 = 1,  /* __half,                              src/ops/all_reduce_fusion.cpp:14-17 */
+    TDE_F32 = 2   /* float,                               src/ops/all_reduce_fusion.cpp:29-33 */
+} tde_dtype;
+
+typedef enum tde_quant {
+    TDE_QUANT_NONE = 0,      /* normed output in the input dtype (the reference's only mode) */
+    TDE_QUANT_FP8_TOKEN = 1, /* OCP e4m3 codes, one fp32 scale per row:  scale = rowamax/448 */
+    TDE_QUANT_FP8_GROUP = 2, /* OCP e4m3 codes, one fp32 scale per [row, 128-column group]  */
+    TDE_QUANT_INT8_TOKEN = 3 /* int8 codes, one fp32 scale per row:      scale = rowamax/127 */
+} tde_quant;
+
+typedef enum tde_algo {
+    TDE_ALGO_AUTO = 0,   /* = TDE_ALGO_FUSED */
+    TDE_ALGO_FUSED = 1,  /* one pass per row: reduce -> residual -> norm -> quant, row kept in registers
+                            (the arithmetic of the one-shot body, impl.h:450-471) */
+    TDE_ALGO_STAGED = 2  /* two launches: (A) N-way reduce of every row into `stage` (impl.h:365-377),
+                            (B) residual + norm (+quant) reading `stage` (impl.h:381-393) */
+} tde_algo;
+
+/* ---- problem / buffers ---------------------------------------------------------------------- */
+typedef struct tde_problem {
+    int32_t dtype;      /* tde_dtype of partials, residual, gamma, residual_out, norm_out */
+    int32_t nranks;     /* number of partial buffers, {2,4,8} */
+    int32_t rank;       /* index of the caller's own partial (informational; order is always 0..N-1) */
+    int32_t quant;      /* tde_quant */
+    int32_t algo;       /* tde_algo */
+    int32_t write_norm; /* quant modes: also write the T-typed normed row to norm_out (0/1).
+                           TDE_QUANT_NONE always writes norm_out. */
+    int64_t tokens;     /* rows; 0 is allowed (no launch) */
+    int64_t hidden;     /* columns per row */
+    float eps;          /* added to mean(x^2) before the reciprocal square root */
+    int32_t reserved;
+} tde_problem;
+
+typedef struct tde_buffers {
+    /* Device pointers, each a contiguous row-major [tokens, hidden] array of `dtype`.
+       If partial_table is non-null it is a DEVICE array of nranks device pointers (the first
+       nranks entries of the reference's workspace table, src/ops/all_reduce_fusion.cpp:159-162)
+       and the kernel reads the pointers from it; entry `rank` is replaced by partial[rank]
+       when partial[rank] is non-null (the caller's own allreduce_in, never staged). */
+    const void *partial[TDE_MAX_RANKS];
+    const void *const *partial_table;
+    const void *residual_in;
+    void *residual_out;
+    void *norm_out;    /* may be null when quant != NONE and write_norm == 0 */
+    const void *gamma; /* [hidden] of `dtype` */
+    void *q_out;       /* [tokens, hidden] bytes (fp8 e4m3 / int8); null when quant == NONE */
+    float *scale_out;  /* [tokens] or [tokens, hidden/128] fp32; null when quant == NONE */
+    void *stage;       /* [tokens, hidden] of `dtype`; required for TDE_ALGO_STAGED */
+} tde_buffers;
+
+typedef struct tde_plan_out {
+    int32_t algo;            /* algorithm that will run (tde_algo, never AUTO) */
+    int32_t reference_algo;  /* what the reference launcher would pick: 1 = one-shot (tokens <= 128),
+                                2 = two-shot (impl.h:491) */
+    int32_t vec_elems;       /* elements per 16-byte access: 8 (bf16/f16), 4 (f32); impl.h:478 */
+    int32_t block_threads;   /* threads per workgroup (multiple of 64) */
+    int32_t vecs_per_thread; /* 16-byte vectors each thread owns per row */
+    int32_t rows_per_block;  /* rows a workgroup processes side by side (one wave group per row) */
+    int32_t grid_blocks;     /* workgroups launched for the row kernel */
+    int32_t reserved;
+    int64_t algorithmic_bytes; /* (N+1)*T*H*e + H*e + T*H*e + OUT, OUT as documented for the quant mode */
+    int64_t scale_elems;       /* number of fp32 scales written */
+} tde_plan_out;
+
+/* ---- entry points --------------------------------------------------------------------------- */
+
+/* Library / ABI version (TDE_ABI_VERSION of the build). */
+int tde_abi_version(void);
+
+/* Human-readable text for a tde_status. Never null. */
+const char *tde_status_string(int status);
+
+/* HIP error code of the most recent TDE_EHIP on this thread (0 if none). */
+int tde_last_hip_error(void);
+
+/* Pure host: validates the problem exactly as tde_reduce_rms does and reports launch geometry and
+   algorithmic bytes.  Touches no device.  Replaces the shape/nranks asserts and the grid/block/
+   algorithm selection of allreduce_fusion_kernel_launcher (impl.h:476-498, 526-534). */
+int tde_plan(const tde_problem *problem, tde_plan_out *plan);
+
+/* Enqueue the row kernel(s) on `hip_stream` (a hipStream_t, null = default stream) of the current
+   device and return without synchronizing.  Replaces allreduce_rms_fusion_impl<T>
+   (impl.h:500-535) for the arithmetic of one rank; quant outputs extend it. */
+int tde_reduce_rms(const tde_problem *problem, const tde_buffers *buffers, void *hip_stream);
+
+/* Tuning hook for sweeps and tests: force vectors-per-thread (1,2,4), rows per workgroup and a cap
+   on the grid (rows beyond it are covered by a grid-stride loop).  0 restores the automatic choice
+   for that field.  Process-wide, not thread-safe.  No counterpart in the reference, whose
+   launcher hard-codes its geometry (impl.h:481-489). */
+int tde_tune_override(int32_t vecs_per_thread, int32_t rows_per_block, int32_t max_grid);
+
+/* ---- emulated peer workspace ----------------------------------------------------------------
+   One allocation per emulated rank plays the role of that rank's IPC-mapped comm buffer
+   (CommWorkspace, src/ops/all_reduce_fusion.cpp:63-96).  Each slot is 2*slot_bytes large: the
+   first half holds the rank's partial, the second half is the gathered/staged region
+   (comm_bufs[r] + size, impl.h:375,387). */
+typedef struct tde_workspace tde_workspace;
+
+int tde_workspace_create(int32_t nranks, int64_t slot_bytes, tde_workspace **out);
+int tde_workspace_destroy(tde_workspace *ws);
+/* Device pointer of slot r (first half). */
+void *tde_workspace_slot(const tde_workspace *ws, int32_t r);
+/* Device pointer of the stage half of slot r. */
+void *tde_workspace_stage(const tde_workspace *ws, int32_t r);
+int64_t tde_workspace_slot_bytes(const tde_workspace *ws);
+int32_t tde_workspace_nranks(const tde_workspace *ws);
+/* Fill `table` (host array, (3*nranks+5) entries) with the reference's pointer-table layout
+   (src/ops/all_reduce_fusion.cpp:159-169): [0,N) slot pointers, [N,2N) flag regions,
+   [2N,3N) one-shot regions (alias the slots here), then 5 scalar cells. */
+int tde_workspace_fill_table(const tde_workspace *ws, void **table, int32_t entries);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TDE_ABI_H */

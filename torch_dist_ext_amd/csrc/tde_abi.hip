@@ -1,0 +1,284 @@
+// C ABI of libtde_hip.so: validation, launch geometry, kernel dispatch and the emulated peer
+// workspace.  Declarations and the reference interfaces they replace are in include/tde_abi.h.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstring>
+#include <new>
+
+#include "tde_abi.h"
+#include "tde_rows.h"
+
+namespace {
+
+thread_local int g_last_hip_error = 0;
+
+int hip_fail(hipError_t e) {
+    g_last_hip_error = (int)e;
+    return TDE_EHIP;
+}
+
+int elem_bytes(int dtype) {
+    switch (dtype) {
+    case TDE_BF16:
+    case TDE_F16: return 2;
+    case TDE_F32: return 4;
+    }
+    return 0;
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+constexpr int kMaxBlock = 1024;
+
+// Tuning override for sweeps (0 = automatic).
+int g_force_vpt = 0;
+int g_force_rows_per_block = 0;
+int g_force_grid = 0;
+
+int validate(const tde_problem *p, tde::Geometry *geo) {
+    if (p == nullptr) return TDE_EINVAL;
+    const int eb = elem_bytes(p->dtype);
+    if (eb == 0) return TDE_EDTYPE;
+    if (!(p->nranks == 2 || p->nranks == 4 || p->nranks == 8)) return TDE_ENRANKS;
+    if (p->rank < 0 || p->rank >= p->nranks) return TDE_ERANK;
+    if (p->tokens < 0 || p->hidden <= 0) return TDE_ESHAPE;
+    if ((p->hidden * eb) % 16 != 0) return TDE_ESHAPE;
+    if (p->quant < TDE_QUANT_NONE || p->quant > TDE_QUANT_INT8_TOKEN) return TDE_EQUANT;
+    if (p->quant == TDE_QUANT_FP8_GROUP && p->hidden % TDE_QUANT_GROUP != 0) return TDE_EQUANT;
+    if (p->algo < TDE_ALGO_AUTO || p->algo > TDE_ALGO_STAGED) return TDE_EALGO;
+    const int vec = 16 / eb;
+    const int64_t nvec = p->hidden / vec;
+    if (nvec > kMaxBlock) return TDE_EHIDDEN; // as the reference: one 16-byte vector per thread, 1024 threads
+    if (p->tokens > 0 && p->tokens * p->hidden / p->hidden != p->tokens) return TDE_ESHAPE;
+
+    // Vectors per thread (1, 2 or 4); a row then needs ceil(nvec/vpt) lanes <= 1024/vpt.
+    int vpt = 1;
+    if (g_force_vpt == 1 || g_force_vpt == 2 || g_force_vpt == 4) vpt = g_force_vpt;
+    const int64_t lanes = (nvec + vpt - 1) / vpt;
+    const int tpr = (int)((lanes + 63) / 64 * 64);
+    int rpb = 256 / tpr; // pack short rows so a workgroup has at least four wavefronts
+    if (rpb < 1) rpb = 1;
+    if (g_force_rows_per_block > 0 && g_force_rows_per_block * tpr <= kMaxBlock / vpt) rpb = g_force_rows_per_block;
+    if (p->tokens > 0 && rpb > p->tokens) rpb = (int)p->tokens;
+    int64_t grid = (p->tokens + rpb - 1) / rpb;
+    if (g_force_grid > 0 && grid > g_force_grid) grid = g_force_grid;
+    if (grid > 0x7fffffff) return TDE_ESHAPE;
+
+    if (geo) {
+        geo->vec_elems = vec;
+        geo->nvec = (int)nvec;
+        geo->vpt = vpt;
+        geo->threads_per_row = tpr;
+        geo->rows_per_block = rpb;
+        geo->block_threads = tpr * rpb;
+        geo->grid = grid;
+    }
+    return TDE_OK;
+}
+
+int64_t algorithmic_bytes(const tde_problem *p, int64_t *scale_elems) {
+    const int64_t e = elem_bytes(p->dtype);
+    const int64_t T = p->tokens, H = p->hidden, N = p->nranks;
+    int64_t out = 0, scales = 0;
+    switch (p->quant) {
+    case TDE_QUANT_NONE: out = T * H * e; break;
+    case TDE_QUANT_FP8_TOKEN:
+    case TDE_QUANT_INT8_TOKEN: scales = T; out = T * H + 4 * scales; break;
+    case TDE_QUANT_FP8_GROUP: scales = T * (H / TDE_QUANT_GROUP); out = T * H + 4 * scales; break;
+    }
+    if (p->quant != TDE_QUANT_NONE && p->write_norm) out += T * H * e;
+    if (scale_elems) *scale_elems = scales;
+    return (N + 1) * T * H * e + H * e + T * H * e + out;
+}
+
+} // namespace
+
+struct tde_workspace {
+    int32_t nranks;
+    int64_t slot_bytes;
+    void *slots[TDE_MAX_RANKS];
+    void *flags;   // nranks regions of 256*nranks ints, zeroed (layout parity only)
+    int32_t *cells; // 5 int cells: counter, two-shot clock, one-shot clock, one-shot size, one-shot clear
+};
+
+extern "C" {
+
+int tde_abi_version(void) { return TDE_ABI_VERSION; }
+
+const char *tde_status_string(int status) {
+    switch (status) {
+    case TDE_OK: return "ok";
+    case TDE_EINVAL: return "invalid argument (null pointer or malformed struct)";
+    case TDE_ENRANKS: return "nranks must be 2, 4 or 8";
+    case TDE_EDTYPE: return "unsupported dtype (bf16, f16, f32)";
+    case TDE_ESHAPE: return "bad shape: hidden*elem_size must be a positive multiple of 16 bytes, tokens >= 0";
+    case TDE_EHIDDEN: return "hidden too large for the one-pass row kernel (max 1024 16-byte vectors per row: 8192 bf16/f16, 4096 f32)";
+    case TDE_EALIGN: return "buffer not 16-byte aligned";
+    case TDE_EQUANT: return "bad quant mode, or per-group quant with hidden not a multiple of 128";
+    case TDE_EALGO: return "bad algorithm, or staged algorithm without a stage buffer";
+    case TDE_EHIP: return "HIP runtime error (see tde_last_hip_error)";
+    case TDE_ERANK: return "rank outside [0, nranks)";
+    case TDE_ENOMEM: return "device allocation failed";
+    }
+    return "unknown status";
+}
+
+int tde_last_hip_error(void) { return g_last_hip_error; }
+
+int tde_tune_override(int32_t vecs_per_thread, int32_t rows_per_block, int32_t max_grid) {
+    g_force_vpt = vecs_per_thread;
+    g_force_rows_per_block = rows_per_block;
+    g_force_grid = max_grid;
+    return TDE_OK;
+}
+
+int tde_plan(const tde_problem *problem, tde_plan_out *plan) {
+    if (plan == nullptr) return TDE_EINVAL;
+    tde::Geometry g{};
+    const int st = validate(problem, &g);
+    if (st != TDE_OK) return st;
+    std::memset(plan, 0, sizeof(*plan));
+    plan->algo = (problem->algo == TDE_ALGO_STAGED) ? TDE_ALGO_STAGED : TDE_ALGO_FUSED;
+    plan->reference_algo = (problem->tokens <= 128) ? 1 : 2;
+    plan->vec_elems = g.vec_elems;
+    plan->block_threads = g.block_threads;
+    plan->vecs_per_thread = g.vpt;
+    plan->rows_per_block = g.rows_per_block;
+    plan->grid_blocks = (int32_t)g.grid;
+    plan->algorithmic_bytes = algorithmic_bytes(problem, &plan->scale_elems);
+    return TDE_OK;
+}
+
+int tde_reduce_rms(const tde_problem *p, const tde_buffers *b, void *hip_stream) {
+    tde::Geometry g{};
+    const int st = validate(p, &g);
+    if (st != TDE_OK) return st;
+    if (b == nullptr) return TDE_EINVAL;
+    const bool quant = p->quant != TDE_QUANT_NONE;
+    const bool wn = !quant || p->write_norm != 0;
+    const bool staged = p->algo == TDE_ALGO_STAGED;
+
+    for (int r = 0; r < p->nranks; ++r) {
+        if (b->partial[r] == nullptr && b->partial_table == nullptr) return TDE_EINVAL;
+        if (!aligned16(b->partial[r])) return TDE_EALIGN;
+    }
+    if (!b->residual_in || !b->residual_out || !b->gamma) return TDE_EINVAL;
+    if (wn && !b->norm_out) return TDE_EINVAL;
+    if (quant && (!b->q_out || !b->scale_out)) return TDE_EINVAL;
+    if (staged && !b->stage) return TDE_EALGO;
+    if (!aligned16(b->residual_in) || !aligned16(b->residual_out) || !aligned16(b->gamma) ||
+        !aligned16(b->norm_out) || !aligned16(b->stage) || !aligned16(b->partial_table))
+        return TDE_EALIGN;
+    if (quant && ((reinterpret_cast<uintptr_t>(b->q_out) & 7u) || (reinterpret_cast<uintptr_t>(b->scale_out) & 3u)))
+        return TDE_EALIGN;
+    if (p->tokens == 0) return TDE_OK;
+
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    tde::RowArgs a{};
+    for (int r = 0; r < p->nranks; ++r) a.part[r] = b->partial[r];
+    a.table = b->partial_table;
+    a.residual_in = b->residual_in;
+    a.residual_out = b->residual_out;
+    a.norm_out = b->norm_out;
+    a.gamma = b->gamma;
+    a.q_out = b->q_out;
+    a.scale_out = b->scale_out;
+    a.stage_out = b->stage;
+    a.tokens = p->tokens;
+    a.hidden = (int32_t)p->hidden;
+    a.nvec = g.nvec;
+    a.threads_per_row = g.threads_per_row;
+    a.rows_per_block = g.rows_per_block;
+    a.eps = p->eps;
+    a.hidden_f = (float)p->hidden;
+
+    int n = p->nranks;
+    hipError_t e = hipSuccess;
+    if (staged) {
+        const int64_t total_vecs = p->tokens * (int64_t)g.nvec;
+        switch (p->dtype) {
+        case TDE_BF16: e = tde::launch_reduce_bf16(n, a, total_vecs, stream); break;
+        case TDE_F16: e = tde::launch_reduce_f16(n, a, total_vecs, stream); break;
+        case TDE_F32: e = tde::launch_reduce_f32(n, a, total_vecs, stream); break;
+        }
+        if (e != hipSuccess) return hip_fail(e);
+        for (int r = 0; r < tde::kMaxKernelRanks; ++r) a.part[r] = nullptr;
+        a.part[0] = b->stage;
+        a.table = nullptr;
+        n = 0;
+    }
+    switch (p->dtype) {
+    case TDE_BF16: e = tde::launch_rows_bf16(n, g.vpt, p->quant, wn, a, g, stream); break;
+    case TDE_F16: e = tde::launch_rows_f16(n, g.vpt, p->quant, wn, a, g, stream); break;
+    case TDE_F32: e = tde::launch_rows_f32(n, g.vpt, p->quant, wn, a, g, stream); break;
+    }
+    if (e != hipSuccess) return hip_fail(e);
+    return TDE_OK;
+}
+
+// ---- emulated peer workspace ----------------------------------------------------------------
+
+int tde_workspace_create(int32_t nranks, int64_t slot_bytes, tde_workspace **out) {
+    if (out == nullptr) return TDE_EINVAL;
+    *out = nullptr;
+    if (!(nranks == 2 || nranks == 4 || nranks == 8)) return TDE_ENRANKS;
+    if (slot_bytes <= 0 || slot_bytes % 16 != 0) return TDE_ESHAPE;
+    tde_workspace *ws = new (std::nothrow) tde_workspace();
+    if (ws == nullptr) return TDE_ENOMEM;
+    ws->nranks = nranks;
+    ws->slot_bytes = slot_bytes;
+    hipError_t e = hipSuccess;
+    for (int r = 0; r < nranks && e == hipSuccess; ++r) e = hipMalloc(&ws->slots[r], (size_t)slot_bytes * 2);
+    const size_t flag_bytes = (size_t)nranks * 256 * nranks * sizeof(int32_t);
+    if (e == hipSuccess) e = hipMalloc(&ws->flags, flag_bytes);
+    if (e == hipSuccess) e = hipMemset(ws->flags, 0, flag_bytes);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ws->cells), 5 * 64);
+    if (e == hipSuccess) e = hipMemset(ws->cells, 0, 5 * 64);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (e != hipSuccess) {
+        tde_workspace_destroy(ws);
+        g_last_hip_error = (int)e;
+        return (e == hipErrorOutOfMemory) ? TDE_ENOMEM : TDE_EHIP;
+    }
+    *out = ws;
+    return TDE_OK;
+}
+
+int tde_workspace_destroy(tde_workspace *ws) {
+    if (ws == nullptr) return TDE_OK;
+    for (int r = 0; r < TDE_MAX_RANKS; ++r)
+        if (ws->slots[r]) (void)hipFree(ws->slots[r]);
+    if (ws->flags) (void)hipFree(ws->flags);
+    if (ws->cells) (void)hipFree(ws->cells);
+    delete ws;
+    return TDE_OK;
+}
+
+void *tde_workspace_slot(const tde_workspace *ws, int32_t r) {
+    if (ws == nullptr || r < 0 || r >= ws->nranks) return nullptr;
+    return ws->slots[r];
+}
+
+void *tde_workspace_stage(const tde_workspace *ws, int32_t r) {
+    if (ws == nullptr || r < 0 || r >= ws->nranks) return nullptr;
+    return static_cast<char *>(ws->slots[r]) + ws->slot_bytes;
+}
+
+int64_t tde_workspace_slot_bytes(const tde_workspace *ws) { return ws ? ws->slot_bytes : 0; }
+int32_t tde_workspace_nranks(const tde_workspace *ws) { return ws ? ws->nranks : 0; }
+
+int tde_workspace_fill_table(const tde_workspace *ws, void **table, int32_t entries) {
+    if (ws == nullptr || table == nullptr) return TDE_EINVAL;
+    const int n = ws->nranks;
+    if (entries != 3 * n + 5) return TDE_EINVAL;
+    for (int r = 0; r < n; ++r) {
+        table[r] = ws->slots[r];
+        table[n + r] = static_cast<char *>(ws->flags) + (size_t)r * 256 * n * sizeof(int32_t);
+        table[2 * n + r] = ws->slots[r];
+    }
+    for (int c = 0; c < 5; ++c) table[3 * n + c] = reinterpret_cast<char *>(ws->cells) + 64 * c;
+    return TDE_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,512 @@
+// Row kernels for gfx950 (MI355X): N-way partial reduce + residual add + RMSNorm + dynamic quant,
+// one pass per row with the row held in registers.
+//
+// Arithmetic contract (what the reference's torch-eager composition computes,
+// test/test_all_reduce_fusion.py:23-28,75-76, with the reduce order of
+// src/common/all_reduce_fusion_impl.h:280-298):
+//   s   = T( ((0 + p_0) + p_1) + ... + p_{N-1} )      fp32 accumulate in rank order, one rounding to T
+//   x   = T( float(s) + float(residual_in) )           -> residual_out            (impl.h:271-278)
+//   rs  = 1 / sqrt( sum(float(x)^2) / H + eps )        fp32, IEEE divide and sqrt
+//   y1  = T( float(x) * rs )
+//   y   = T( float(gamma) * float(y1) )                -> norm_out
+//   per-token fp8 : scale = amax|y| / 448, code = e4m3( clamp(float(y)/scale, +-448) )
+//   per-group fp8 : the same over each 128-column group
+//   per-token int8: scale = amax|y| / 127, code = clamp(rne(float(y)/scale), +-127)
+//
+// Included by one translation unit per element type; nothing here is exported.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "tde_abi.h"
+
+namespace tde {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+constexpr int kMaxWavesPerBlock = 16;
+constexpr int kMaxKernelRanks = 8;
+
+// Kernel argument block (passed by value in kernarg memory).
+struct RowArgs {
+    const void *part[kMaxKernelRanks]; // host-known partial pointers (or the stage buffer in [0])
+    const void *const *table;          // optional device pointer table; entry r used when part[r] == null
+    const void *residual_in;
+    void *residual_out;
+    void *norm_out;
+    const void *gamma;
+    void *q_out;
+    float *scale_out;
+    void *stage_out; // stage A destination
+    int64_t tokens;
+    int32_t hidden;
+    int32_t nvec;           // 16-byte vectors per row
+    int32_t threads_per_row; // multiple of 64
+    int32_t rows_per_block;
+    float eps;
+    float hidden_f;
+};
+
+// ---------------------------------------------------------------------------------------------
+// Element traits: a 16-byte vector <-> VEC floats.  pack() rounds to nearest even.
+// ---------------------------------------------------------------------------------------------
+struct ElemBF16 {
+    static constexpr int VEC = 8;
+    static constexpr int BYTES = 2;
+    static __device__ __forceinline__ void unpack(u32x4 raw, float (&f)[VEC]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __builtin_bit_cast(float, raw[i] << 16);
+            f[2 * i + 1] = __builtin_bit_cast(float, raw[i] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[VEC]) {
+        u32x4 raw;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f32x2 v = {f[2 * i], f[2 * i + 1]};
+            raw[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+        }
+        return raw;
+    }
+};
+
+struct ElemF16 {
+    static constexpr int VEC = 8;
+    static constexpr int BYTES = 2;
+    static __device__ __forceinline__ void unpack(u32x4 raw, float (&f)[VEC]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f16x2 h = __builtin_bit_cast(f16x2, raw[i]);
+            f[2 * i] = (float)h[0];
+            f[2 * i + 1] = (float)h[1];
+        }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[VEC]) {
+        u32x4 raw;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f16x2 h = {(_Float16)f[2 * i], (_Float16)f[2 * i + 1]};
+            raw[i] = __builtin_bit_cast(uint32_t, h);
+        }
+        return raw;
+    }
+};
+
+struct ElemF32 {
+    static constexpr int VEC = 4;
+    static constexpr int BYTES = 4;
+    static __device__ __forceinline__ void unpack(u32x4 raw, float (&f)[VEC]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = __builtin_bit_cast(float, raw[i]);
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[VEC]) {
+        u32x4 raw;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) raw[i] = __builtin_bit_cast(uint32_t, f[i]);
+        return raw;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// 64-lane wavefront reductions: four DPP steps inside each 16-lane row, then the four row
+// results are combined through v_readlane.  Every lane ends with the same value.
+// ---------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+struct OpSum {
+    static __device__ __forceinline__ float f(float a, float b) { return a + b; }
+};
+struct OpMax {
+    static __device__ __forceinline__ float f(float a, float b) { return fmaxf(a, b); }
+};
+
+template <class Op>
+__device__ __forceinline__ float row16_reduce(float v) {
+    v = Op::f(v, dpp_move<0xB1>(v));  // quad_perm [1,0,3,2]
+    v = Op::f(v, dpp_move<0x4E>(v));  // quad_perm [2,3,0,1]
+    v = Op::f(v, dpp_move<0x141>(v)); // row_half_mirror
+    v = Op::f(v, dpp_move<0x140>(v)); // row_mirror
+    return v;
+}
+
+__device__ __forceinline__ float read_lane(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+template <class Op>
+__device__ __forceinline__ float wave_reduce(float v) {
+    v = row16_reduce<Op>(v);
+    const float a = read_lane(v, 0), b = read_lane(v, 16), c = read_lane(v, 32), d = read_lane(v, 48);
+    return Op::f(Op::f(a, b), Op::f(c, d));
+}
+
+// Reduce over the `waves_per_row` wavefronts that share a row.  `slots` is this iteration's LDS
+// buffer indexed by wavefront number inside the block; the caller alternates between two buffers
+// so that one barrier per reduction is enough.  Identity is 0 for both operators as used here
+// (sums of squares and maxima of absolute values).
+template <class Op>
+__device__ __forceinline__ float row_reduce(float v, float *slots, int wave, int lane, int first_wave,
+                                            int waves_per_row) {
+    v = wave_reduce<Op>(v);
+    if (waves_per_row == 1) return v;
+    if (lane == 0) slots[wave] = v;
+    __syncthreads();
+    const int k = lane & 15;
+    const float t = (k < waves_per_row) ? slots[first_wave + k] : 0.0f;
+    return row16_reduce<Op>(t);
+}
+
+// Streaming (non-temporal) 128-bit access at a wavefront-uniform base plus a 32-bit lane offset:
+// the form that maps to global_load/store_dwordx4 with an SGPR base.
+// Every buffer is device (global) memory, so the accesses are typed as address space 1 and never
+// go through the flat aperture check.
+#define TDE_GLOBAL __attribute__((address_space(1)))
+template <class V>
+__device__ __forceinline__ const TDE_GLOBAL V *global_ptr(const void *base, uint32_t byte_off) {
+    return (const TDE_GLOBAL V *)((const TDE_GLOBAL char *)base + byte_off);
+}
+template <class V>
+__device__ __forceinline__ TDE_GLOBAL V *global_ptr(void *base, uint32_t byte_off) {
+    return (TDE_GLOBAL V *)((TDE_GLOBAL char *)base + byte_off);
+}
+__device__ __forceinline__ u32x4 load_stream(const void *base, uint32_t byte_off) {
+    return __builtin_nontemporal_load(global_ptr<u32x4>(base, byte_off));
+}
+__device__ __forceinline__ void store_stream(void *base, uint32_t byte_off, u32x4 v) {
+    __builtin_nontemporal_store(v, global_ptr<u32x4>(base, byte_off));
+}
+
+// Pack VEC fp32 values (already clamped to +-448) to OCP e4m3 bytes, round to nearest even.
+template <int VEC>
+__device__ __forceinline__ void pack_fp8(const float (&q)[VEC], uint32_t (&out)[VEC / 4]) {
+#pragma unroll
+    for (int w = 0; w < VEC / 4; ++w) {
+        int word = 0;
+        word = __builtin_amdgcn_cvt_pk_fp8_f32(q[4 * w], q[4 * w + 1], word, false);
+        word = __builtin_amdgcn_cvt_pk_fp8_f32(q[4 * w + 2], q[4 * w + 3], word, true);
+        out[w] = (uint32_t)word;
+    }
+}
+
+template <int VEC>
+__device__ __forceinline__ void pack_int8(const float (&q)[VEC], uint32_t (&out)[VEC / 4]) {
+#pragma unroll
+    for (int w = 0; w < VEC / 4; ++w) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int code = (int)__builtin_rintf(q[4 * w + b]); // ties to even
+            word |= ((uint32_t)code & 0xffu) << (8 * b);
+        }
+        out[w] = word;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// The row kernel.
+//   E      element traits
+//   N      number of partials summed per element; N == 0 means "the sum was staged":
+//          part[0] already holds s (a T-typed [tokens,hidden] buffer)
+//   VPT    16-byte vectors per thread per row
+//   Q      tde_quant
+//   WN     write the T-typed normed row (always true for Q == NONE)
+// Block layout: rows_per_block row groups of threads_per_row threads; thread t of a row group
+// owns vectors t, t + threads_per_row, ... (coalesced 1 KiB per wavefront per load).
+// ---------------------------------------------------------------------------------------------
+template <class E, int N, int VPT, int Q, bool WN>
+__global__ void __launch_bounds__(1024 / VPT) row_kernel(const RowArgs a) {
+    constexpr int VEC = E::VEC;
+    constexpr int NP = (N == 0) ? 1 : N;
+    __shared__ float lds_sum[2][kMaxWavesPerBlock];
+    __shared__ float lds_max[2][kMaxWavesPerBlock];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid >> 6;
+    const int tpr = a.threads_per_row;
+    const int waves_per_row = tpr >> 6;
+    const int group = __builtin_amdgcn_readfirstlane(tid / tpr); // uniform inside a wavefront
+    const int t = tid - group * tpr;
+    const int first_wave = group * waves_per_row;
+
+    const void *part[NP];
+#pragma unroll
+    for (int r = 0; r < NP; ++r) {
+        part[r] = a.part[r];
+        if (part[r] == nullptr) part[r] = a.table[r];
+    }
+
+    // gamma is shared by every row this block touches: keep it in registers.
+    u32x4 gamma_raw[VPT];
+    bool col_ok[VPT];
+    uint32_t lane_off[VPT]; // byte offset of this thread's vector j inside a row
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int v = j * tpr + t;
+        col_ok[j] = v < a.nvec;
+        lane_off[j] = (uint32_t)v * 16u;
+        gamma_raw[j] = col_ok[j] ? *global_ptr<u32x4>(a.gamma, lane_off[j]) : u32x4{0, 0, 0, 0};
+    }
+
+    const int64_t row_stride = (int64_t)gridDim.x * a.rows_per_block;
+    int parity = 0;
+    for (int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block; row0 < a.tokens; row0 += row_stride, parity ^= 1) {
+        const int64_t row = row0 + group;
+        const bool row_ok = row < a.tokens;
+        const int64_t row_elem = row * (int64_t)a.hidden;
+        const int64_t row_byte = row_elem * E::BYTES; // wavefront-uniform
+
+        // ---- issue every load of the row before consuming any ---------------------------------
+        u32x4 praw[VPT][NP];
+        u32x4 rraw[VPT];
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+#pragma unroll
+            for (int r = 0; r < NP; ++r) praw[j][r] = u32x4{0, 0, 0, 0};
+            rraw[j] = u32x4{0, 0, 0, 0};
+            if (row_ok && col_ok[j]) {
+#pragma unroll
+                for (int r = 0; r < NP; ++r)
+                    praw[j][r] = load_stream(static_cast<const char *>(part[r]) + row_byte, lane_off[j]);
+                rraw[j] = load_stream(static_cast<const char *>(a.residual_in) + row_byte, lane_off[j]);
+            }
+        }
+
+        // ---- reduce, residual add, sum of squares ------------------------------------------------
+        u32x4 xraw[VPT];
+        float sumsq = 0.0f;
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+            float s[VEC];
+            if constexpr (N == 0) {
+                E::unpack(praw[j][0], s);
+            } else {
+                float acc[VEC];
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+#pragma unroll
+                for (int r = 0; r < NP; ++r) {
+                    float p[VEC];
+                    E::unpack(praw[j][r], p);
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) acc[i] += p[i];
+                }
+                E::unpack(E::pack(acc), s);
+            }
+            float res[VEC], x[VEC];
+            E::unpack(rraw[j], res);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) x[i] = s[i] + res[i];
+            xraw[j] = E::pack(x);
+            const bool ok = row_ok && col_ok[j];
+            if (ok) store_stream(static_cast<char *>(a.residual_out) + row_byte, lane_off[j], xraw[j]);
+            E::unpack(xraw[j], x);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) sumsq += x[i] * x[i];
+        }
+        sumsq = row_reduce<OpSum>(sumsq, lds_sum[parity], wave, lane, first_wave, waves_per_row);
+        const float rs = 1.0f / __builtin_sqrtf(sumsq / a.hidden_f + a.eps);
+
+        // ---- normalize ------------------------------------------------------------------------------
+        u32x4 yraw[VPT];
+        float amax[VPT];
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+            float x[VEC], g[VEC], y[VEC];
+            E::unpack(xraw[j], x);
+            E::unpack(gamma_raw[j], g);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) y[i] = x[i] * rs;
+            E::unpack(E::pack(y), y);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) y[i] = g[i] * y[i];
+            yraw[j] = E::pack(y);
+            const bool ok = row_ok && col_ok[j];
+            if constexpr (Q == TDE_QUANT_NONE || WN) {
+                if (ok) store_stream(static_cast<char *>(a.norm_out) + row_byte, lane_off[j], yraw[j]);
+            }
+            if constexpr (Q != TDE_QUANT_NONE) {
+                E::unpack(yraw[j], y);
+                float m = 0.0f;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) m = fmaxf(m, __builtin_fabsf(y[i]));
+                amax[j] = m;
+            }
+        }
+
+        // ---- dynamic quant epilogue ---------------------------------------------------------------
+        if constexpr (Q != TDE_QUANT_NONE) {
+            constexpr float QMAX = (Q == TDE_QUANT_INT8_TOKEN) ? 127.0f : 448.0f;
+            float scale[VPT];
+            if constexpr (Q == TDE_QUANT_FP8_GROUP) {
+                constexpr int LANES_PER_GROUP = TDE_QUANT_GROUP / VEC; // 16 (2-byte types) or 32 (fp32)
+#pragma unroll
+                for (int j = 0; j < VPT; ++j) {
+                    float m = row16_reduce<OpMax>(amax[j]);
+                    if constexpr (LANES_PER_GROUP == 32) m = fmaxf(m, __shfl_xor(m, 16, kWave));
+                    scale[j] = m / QMAX;
+                    const int v = j * tpr + t;
+                    if (row_ok && col_ok[j] && (lane & (LANES_PER_GROUP - 1)) == 0) {
+                        const int64_t groups_per_row = a.hidden / TDE_QUANT_GROUP;
+                        ((TDE_GLOBAL float *)a.scale_out)[row * groups_per_row + v / LANES_PER_GROUP] = scale[j];
+                    }
+                }
+            } else {
+                float m = amax[0];
+#pragma unroll
+                for (int j = 1; j < VPT; ++j) m = fmaxf(m, amax[j]);
+                m = row_reduce<OpMax>(m, lds_max[parity], wave, lane, first_wave, waves_per_row);
+                const float sc = m / QMAX;
+#pragma unroll
+                for (int j = 0; j < VPT; ++j) scale[j] = sc;
+                if (row_ok && t == 0) ((TDE_GLOBAL float *)a.scale_out)[row] = sc;
+            }
+#pragma unroll
+            for (int j = 0; j < VPT; ++j) {
+                float y[VEC], q[VEC];
+                E::unpack(yraw[j], y);
+                const float div = (scale[j] > 0.0f) ? scale[j] : 1.0f;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) q[i] = fminf(fmaxf(y[i] / div, -QMAX), QMAX);
+                uint32_t codes[VEC / 4];
+                if constexpr (Q == TDE_QUANT_INT8_TOKEN)
+                    pack_int8<VEC>(q, codes);
+                else
+                    pack_fp8<VEC>(q, codes);
+                if (row_ok && col_ok[j]) {
+                    char *dst = static_cast<char *>(a.q_out) + row_elem;
+                    const uint32_t code_off = (lane_off[j] / 16u) * (uint32_t)VEC;
+                    if constexpr (VEC == 8) {
+                        u32x2 w = {codes[0], codes[1]};
+                        __builtin_nontemporal_store(w, global_ptr<u32x2>(dst, code_off));
+                    } else {
+                        __builtin_nontemporal_store(codes[0], global_ptr<uint32_t>(dst, code_off));
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Stage A of the staged algorithm: s = T(sum of partials) for every element, no row structure.
+template <class E, int N>
+__global__ void __launch_bounds__(256) reduce_kernel(const RowArgs a, int64_t total_vecs) {
+    constexpr int VEC = E::VEC;
+    const void *part[N];
+#pragma unroll
+    for (int r = 0; r < N; ++r) {
+        part[r] = a.part[r];
+        if (part[r] == nullptr) part[r] = a.table[r];
+    }
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < total_vecs; v += stride) {
+        u32x4 raw[N];
+#pragma unroll
+        for (int r = 0; r < N; ++r)
+            raw[r] = __builtin_nontemporal_load((const TDE_GLOBAL u32x4 *)((const TDE_GLOBAL char *)part[r] + v * 16));
+        float acc[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+#pragma unroll
+        for (int r = 0; r < N; ++r) {
+            float p[VEC];
+            E::unpack(raw[r], p);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] += p[i];
+        }
+        // The staged sum is re-read by stage B right away: ordinary (cacheable) store.
+        *(TDE_GLOBAL u32x4 *)((TDE_GLOBAL char *)a.stage_out + v * 16) = E::pack(acc);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Host-side launch geometry shared by tde_plan and the launchers.
+// ---------------------------------------------------------------------------------------------
+struct Geometry {
+    int vec_elems;
+    int nvec;
+    int vpt;
+    int threads_per_row;
+    int rows_per_block;
+    int block_threads;
+    int64_t grid;
+};
+
+// Per-dtype launchers, defined in tde_rows_<dtype>.hip.
+hipError_t launch_rows_bf16(int n, int vpt, int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s);
+hipError_t launch_rows_f16(int n, int vpt, int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s);
+hipError_t launch_rows_f32(int n, int vpt, int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s);
+hipError_t launch_reduce_bf16(int n, const RowArgs &a, int64_t total_vecs, hipStream_t s);
+hipError_t launch_reduce_f16(int n, const RowArgs &a, int64_t total_vecs, hipStream_t s);
+hipError_t launch_reduce_f32(int n, const RowArgs &a, int64_t total_vecs, hipStream_t s);
+
+// Instantiation + dispatch body used by the three per-dtype translation units.
+template <class E, int N, int VPT>
+hipError_t launch_rows_nv(int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s) {
+    const dim3 grid((unsigned)g.grid), block((unsigned)g.block_threads);
+#define TDE_LAUNCH(QM, WNB)                                                   \
+    hipLaunchKernelGGL((row_kernel<E, N, VPT, QM, WNB>), grid, block, 0, s, a); \
+    return hipGetLastError();
+    switch (q) {
+    case TDE_QUANT_NONE: TDE_LAUNCH(TDE_QUANT_NONE, true)
+    case TDE_QUANT_FP8_TOKEN:
+        if (wn) { TDE_LAUNCH(TDE_QUANT_FP8_TOKEN, true) } else { TDE_LAUNCH(TDE_QUANT_FP8_TOKEN, false) }
+    case TDE_QUANT_FP8_GROUP:
+        if (wn) { TDE_LAUNCH(TDE_QUANT_FP8_GROUP, true) } else { TDE_LAUNCH(TDE_QUANT_FP8_GROUP, false) }
+    case TDE_QUANT_INT8_TOKEN:
+        if (wn) { TDE_LAUNCH(TDE_QUANT_INT8_TOKEN, true) } else { TDE_LAUNCH(TDE_QUANT_INT8_TOKEN, false) }
+    }
+#undef TDE_LAUNCH
+    return hipErrorInvalidValue;
+}
+
+template <class E, int N>
+hipError_t launch_rows_n(int vpt, int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s) {
+    switch (vpt) {
+    case 1: return launch_rows_nv<E, N, 1>(q, wn, a, g, s);
+    case 2: return launch_rows_nv<E, N, 2>(q, wn, a, g, s);
+    case 4: return launch_rows_nv<E, N, 4>(q, wn, a, g, s);
+    }
+    return hipErrorInvalidValue;
+}
+
+template <class E>
+hipError_t launch_rows_e(int n, int vpt, int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s) {
+    switch (n) {
+    case 0: return launch_rows_n<E, 0>(vpt, q, wn, a, g, s);
+    case 2: return launch_rows_n<E, 2>(vpt, q, wn, a, g, s);
+    case 4: return launch_rows_n<E, 4>(vpt, q, wn, a, g, s);
+    case 8: return launch_rows_n<E, 8>(vpt, q, wn, a, g, s);
+    }
+    return hipErrorInvalidValue;
+}
+
+template <class E>
+hipError_t launch_reduce_e(int n, const RowArgs &a, int64_t total_vecs, hipStream_t s) {
+    if (total_vecs <= 0) return hipSuccess;
+    const int block = 256;
+    int64_t blocks = (total_vecs + block - 1) / block;
+    const int64_t cap = 256 * 16; // 16 workgroups of 4 wavefronts per CU, grid-stride beyond that
+    if (blocks > cap) blocks = cap;
+    const dim3 grid((unsigned)blocks), blk(block);
+    switch (n) {
+    case 2: hipLaunchKernelGGL((reduce_kernel<E, 2>), grid, blk, 0, s, a, total_vecs); break;
+    case 4: hipLaunchKernelGGL((reduce_kernel<E, 4>), grid, blk, 0, s, a, total_vecs); break;
+    case 8: hipLaunchKernelGGL((reduce_kernel<E, 8>), grid, blk, 0, s, a, total_vecs); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+} // namespace tde
