@@ -29,8 +29,18 @@ GROUP = 128
 
 
 def reduce_residual(parts: torch.Tensor, residual_in: torch.Tensor) -> torch.Tensor:
-    """parts [N,T,H], residual_in [T,H], both dtype T.  test_all_reduce_fusion.py:75."""
-    return parts.sum(dim=0) + residual_in
+    """parts [N,T,H], residual_in [T,H], both dtype T.
+
+    test_all_reduce_fusion.py:75 writes `allreduce_in.sum(dim=0) + residual_in`.  The sum is restated as
+    what the kernel contract fixes (all_reduce_fusion_impl.h:280-298): fp32 accumulation in rank order
+    0..N-1, one rounding to T.  torch's CPU `sum(dim=0)` is bit-identical to this wherever it runs its
+    vectorized path; only the last few elements of the flattened tensor (the scalar tail when T*H is
+    not a multiple of its vector chunk) are added in a different, host-ISA-dependent order
+    (tests/test_oracle.py::test_torch_sum_dim0_is_rank_order_except_flat_tail)."""
+    acc = torch.zeros(parts.shape[1:], dtype=torch.float32)
+    for r in range(parts.shape[0]):
+        acc = acc + parts[r].float()
+    return acc.to(parts.dtype) + residual_in
 
 
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:

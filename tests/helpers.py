@@ -84,31 +84,106 @@ def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, wri
     return out
 
 
-def check_against_oracle(got, want, quant, norm_ulp=1, scale_rtol=1e-6, allow_scale_outliers=0):
-    """The parity bar: residual bit-exact, normed within norm_ulp units in the last place, codes within
-    one quant step, scales within scale_rtol relative.  Returns a dict of mismatch statistics."""
+def _rs_candidates(x, eps, span):
+    """Per-row reciprocal RMS exactly as the eager composition computes it, plus its fp32 neighbours
+    up to `span` units in the last place on either side: list of [T,1] fp32 tensors."""
+    variance = x.float().pow(2).mean(-1, keepdim=True)
+    rs0 = torch.rsqrt(variance + eps)
+    out = [rs0]
+    up = down = rs0
+    for _ in range(span):
+        up = torch.nextafter(up, torch.full_like(up, float("inf")))
+        down = torch.nextafter(down, torch.zeros_like(down))
+        out += [up, down]
+    return out
+
+
+def norm_rows_explained(norm_got, residual_out, gamma, eps, span=4):
+    """Row by row: is the kernel's normed row bit-identical to the eager composition
+    ((x*rs).to(T) then weight*x, test/test_all_reduce_fusion.py:25-28) evaluated with a reciprocal RMS
+    within `span` fp32 ulps of the oracle's?  The only freedom this leaves the kernel is the summation
+    order of the fp32 mean of squares, which torch's CPU kernel does not pin either (it depends on the
+    host's vector width).  Returns (all_rows_ok, index of the candidate each row matched or -1)."""
+    x = residual_out
+    T = x.shape[0]
+    matched = torch.full((T,), -1, dtype=torch.int64)
+    for k, rs in enumerate(_rs_candidates(x, eps, span)):
+        y = gamma * (x * rs).to(x.dtype)
+        same = (y.view(torch.uint8).view(T, -1) == norm_got.view(torch.uint8).view(T, -1)).all(dim=1)
+        matched = torch.where((matched < 0) & same, torch.full_like(matched, k), matched)
+    return bool((matched >= 0).all()), matched
+
+
+def quant_from_own_norm(norm_got, quant):
+    """The oracle's quantizer applied to the kernel's own normed rows."""
+    from oracle import eager
+    if quant == "fp8_token":
+        return eager.quant_fp8(norm_got, None)
+    if quant == "fp8_group":
+        return eager.quant_fp8(norm_got, eager.GROUP)
+    return eager.quant_int8(norm_got)
+
+
+def check_against_oracle(got, want, quant, gamma=None, eps=None, norm_ulp=2, norm_flip_frac=2e-4, scale_rtol=1e-6):
+    """Two levels.
+
+    Stage-exact (needs gamma/eps and a norm_out from the kernel):
+      residual_out bit-exact; every normed row bit-identical to the eager composition for a reciprocal
+      RMS within 4 fp32 ulps of the oracle's; scales and codes bit-identical to the oracle's quantizer
+      applied to the kernel's own normed rows.
+    End to end against the oracle's outputs:
+      normed within 1 ulp except a fraction <= norm_flip_frac of elements (never more than norm_ulp):
+      those are elements whose first rounding lands on the other side because the reciprocal RMS
+      differs in its last fp32 bit; codes within one quant step; scales within scale_rtol relative,
+      except rows/groups whose maximum element is one of those flipped elements (counted, and bounded
+      by the number of flipped elements).
+    Returns mismatch statistics."""
     stats = {}
     assert bits_equal(got["residual_out"], want["residual_out"]), "residual_out is not bit-exact"
+    flipped = 0
     if "norm_out" in got:
-        d = ulp_distance(got["norm_out"], want["norm_out"])
-        stats["norm_max_ulp"] = int(d.max()) if d.numel() else 0
-        stats["norm_mismatch_frac"] = float((d > 0).float().mean()) if d.numel() else 0.0
-        assert stats["norm_max_ulp"] <= norm_ulp, "norm_out off by %d ulp" % stats["norm_max_ulp"]
         assert not torch.isnan(got["norm_out"].float()).any()
+        d = ulp_distance(got["norm_out"], want["norm_out"])
+        n = max(d.numel(), 1)
+        flipped = int((d > 0).sum())
+        stats["norm_max_ulp"] = int(d.max()) if d.numel() else 0
+        stats["norm_diff_elems"] = flipped
+        stats["norm_gt1_elems"] = int((d > 1).sum())
+        if got["norm_out"].dtype == torch.float32:
+            # fp32 has no second rounding to absorb a last-bit difference of the reciprocal RMS: whole rows
+            # move by an ulp or two.  End to end the reference's own tolerance applies (atol 1e-4,
+            # test/unit_test.cpp:219); the stage-exact check below stays bit-exact.
+            assert stats["norm_max_ulp"] <= 8
+            assert float((got["norm_out"] - want["norm_out"]).abs().max()) <= 1e-4
+            flipped = got["norm_out"].shape[0]
+        else:
+            assert stats["norm_max_ulp"] <= norm_ulp, "norm_out off by %d ulp" % stats["norm_max_ulp"]
+            assert flipped / n <= norm_flip_frac, "%d of %d normed elements differ" % (flipped, n)
+        if gamma is not None:
+            ok, matched = norm_rows_explained(got["norm_out"], got["residual_out"], gamma, eps)
+            stats["rows_needing_rs_neighbour"] = int((matched > 0).sum())
+            assert ok, "%d normed rows are not the eager composition for any reciprocal RMS within 4 ulps" % int(
+                (matched < 0).sum())
     if quant != "none":
+        if "norm_out" in got:
+            q_own, s_own = quant_from_own_norm(got["norm_out"], quant)
+            assert bits_equal(got["scale"].reshape(-1), s_own.reshape(-1)), "scales differ from amax(own normed rows)/qmax"
+            assert bits_equal(got["q"], q_own), "codes differ from the oracle quantizer applied to the kernel's normed rows"
+            stats["quant_stage_exact"] = True
         gs, ws = got["scale"].double().flatten(), want["scale"].double().flatten()
         rel = (gs - ws).abs() / ws.abs().clamp_min(1e-30)
         rel = torch.where((gs == 0) & (ws == 0), torch.zeros_like(rel), rel)
         bad = int((rel > scale_rtol).sum())
         stats["scale_max_rel"] = float(rel.max()) if rel.numel() else 0.0
         stats["scale_bad"] = bad
-        assert bad <= allow_scale_outliers, "%d scales differ by more than %g relative (max %g)" % (
-            bad, scale_rtol, stats["scale_max_rel"])
+        assert bad <= flipped, "%d scales differ by more than %g relative (max %g) with only %d flipped elements" % (
+            bad, scale_rtol, stats["scale_max_rel"], flipped)
+        assert stats["scale_max_rel"] <= 2.0 ** -7, "a scale is off by more than one ulp of the element type"
         if quant == "int8_token":
             dq = (got["q"].to(torch.int32) - want["q"].to(torch.int32)).abs()
         else:
             dq = ulp_distance(got["q"], want["q"])
         stats["q_max_step"] = int(dq.max()) if dq.numel() else 0
-        stats["q_mismatch_frac"] = float((dq > 0).float().mean()) if dq.numel() else 0.0
+        stats["q_diff_elems"] = int((dq > 0).sum())
         assert stats["q_max_step"] <= 1, "codes off by %d quant steps" % stats["q_max_step"]
     return stats

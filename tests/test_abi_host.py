@@ -1,0 +1,176 @@
+"""CPU-only checks of the boundary: the C-ABI library loads and exports every symbol the header
+declares, tde_plan validates like the reference's launcher asserts, algorithmic bytes match the
+documented formula, and the torch layer registers the reference's schemas verbatim."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from torch_dist_ext_amd import _capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "tde_abi.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tde_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_capi.LIB_PATH)
+    declared = _declared_functions()
+    assert len(declared) >= 12
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert sorted(_capi.EXPORTS) == declared
+    assert _capi.load().tde_abi_version() == 1
+
+
+def test_struct_layouts_match_header():
+    assert ctypes.sizeof(_capi.Problem) == 48
+    assert ctypes.sizeof(_capi.Buffers) == (16 + 8) * 8
+    assert ctypes.sizeof(_capi.PlanOut) == 48
+
+
+def _plan(**kw):
+    base = dict(dtype=_capi.BF16, nranks=8, tokens=2048, hidden=8192, eps=1e-5)
+    base.update(kw)
+    return _capi.plan(_capi.make_problem(**base))
+
+
+@pytest.mark.parametrize("kw,status", [
+    (dict(nranks=3), _capi.ENRANKS), (dict(nranks=16), _capi.ENRANKS), (dict(nranks=1), _capi.ENRANKS),
+    (dict(dtype=7), _capi.EDTYPE),
+    (dict(hidden=8190), _capi.ESHAPE),      # 8190*2 bytes is not a multiple of 16 (impl.h:480)
+    (dict(hidden=0), _capi.ESHAPE), (dict(tokens=-1), _capi.ESHAPE),
+    (dict(hidden=8200), _capi.EHIDDEN),     # beyond 1024 vectors per row (the reference asserts hidden <= 8192)
+    (dict(dtype=_capi.F32, hidden=4100), _capi.EHIDDEN),
+    (dict(quant=9), _capi.EQUANT), (dict(quant=_capi.QUANT_FP8_GROUP, hidden=1032), _capi.EQUANT),
+    (dict(algo=5), _capi.EALGO), (dict(rank=8), _capi.ERANK), (dict(rank=-1), _capi.ERANK),
+])
+def test_plan_rejects(kw, status):
+    with pytest.raises(_capi.TdeError) as e:
+        _plan(**kw)
+    assert e.value.status == status
+    assert _capi.status_string(status) != "unknown status"
+
+
+def test_plan_null_pointers():
+    lib = _capi.load()
+    assert lib.tde_plan(None, None) == _capi.EINVAL
+    assert lib.tde_reduce_rms(None, None, None) == _capi.EINVAL
+    out = _capi.PlanOut()
+    assert lib.tde_plan(None, ctypes.byref(out)) == _capi.EINVAL
+
+
+@pytest.mark.parametrize("cfg,expected", [
+    # BASELINE configs: bytes = (N+1)*T*H*e + H*e + T*H*e + OUT
+    (dict(nranks=2, tokens=16, hidden=1024, quant=_capi.QUANT_NONE), 165888),
+    (dict(nranks=8, tokens=128, hidden=4096, quant=_capi.QUANT_NONE), 11542528),
+    (dict(nranks=8, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_TOKEN), 352346112),
+    (dict(nranks=4, tokens=8192, hidden=7168, quant=_capi.QUANT_FP8_GROUP), 765212672),
+    (dict(dtype=_capi.F16, nranks=4, tokens=32768, hidden=5120, quant=_capi.QUANT_INT8_TOKEN), 66564 * 32768 + 10240),
+    (dict(dtype=_capi.F16, nranks=4, tokens=1, hidden=5120, quant=_capi.QUANT_INT8_TOKEN), 66564 + 10240),
+])
+def test_algorithmic_bytes(cfg, expected):
+    assert _plan(**cfg).algorithmic_bytes == expected
+
+
+def test_plan_geometry_and_reference_threshold():
+    p = _plan(tokens=128)
+    assert p.reference_algo == 1 and _plan(tokens=129).reference_algo == 2   # kOneShotMaxToken, impl.h:24,491
+    assert p.vec_elems == 8 and _plan(dtype=_capi.F32, hidden=1024).vec_elems == 4
+    for hidden in (124, 508, 1024, 4096, 5120, 7168, 8192):
+        for dt in (_capi.BF16, _capi.F32):
+            if (dt == _capi.F32 and hidden > 4096) or (dt == _capi.BF16 and hidden % 8):
+                continue
+            q = _plan(dtype=dt, hidden=hidden, tokens=777)
+            nvec = hidden // q.vec_elems
+            assert q.block_threads % 64 == 0 and q.block_threads <= 1024
+            per_row = q.block_threads // q.rows_per_block
+            assert per_row * q.vecs_per_thread >= nvec                  # every vector of a row has an owner
+            assert q.grid_blocks * q.rows_per_block >= 777
+    assert _plan(tokens=0).grid_blocks == 0
+    assert _plan(algo=_capi.ALGO_STAGED).algo == _capi.ALGO_STAGED and _plan().algo == _capi.ALGO_FUSED
+    assert _plan(quant=_capi.QUANT_FP8_GROUP, hidden=7168, nranks=4, tokens=8192).scale_elems == 8192 * 56
+
+
+def test_reduce_rms_argument_checks_need_no_gpu():
+    lib = _capi.load()
+    prob = _capi.make_problem(_capi.BF16, 2, 4, 256, 1e-6)
+    b = _capi.Buffers()
+    assert lib.tde_reduce_rms(ctypes.byref(prob), ctypes.byref(b), None) == _capi.EINVAL      # no partials
+    b.partial[0], b.partial[1] = 0x1000, 0x2008                                                   # misaligned
+    assert lib.tde_reduce_rms(ctypes.byref(prob), ctypes.byref(b), None) == _capi.EALIGN
+    b.partial[1] = 0x2000
+    assert lib.tde_reduce_rms(ctypes.byref(prob), ctypes.byref(b), None) == _capi.EINVAL      # no residual/gamma
+    b.residual_in = b.residual_out = b.gamma = b.norm_out = 0x3000
+    prob.algo = _capi.ALGO_STAGED
+    assert lib.tde_reduce_rms(ctypes.byref(prob), ctypes.byref(b), None) == _capi.EALGO       # staged without stage
+    prob.algo = _capi.ALGO_AUTO
+    prob.quant = _capi.QUANT_FP8_TOKEN
+    assert lib.tde_reduce_rms(ctypes.byref(prob), ctypes.byref(b), None) == _capi.EINVAL      # quant without q/scale
+    prob.quant = _capi.QUANT_NONE
+    prob.tokens = 0
+    assert lib.tde_reduce_rms(ctypes.byref(prob), ctypes.byref(b), None) == _capi.OK          # empty input: no launch
+
+
+def test_workspace_argument_checks_need_no_gpu():
+    lib = _capi.load()
+    ws = ctypes.c_void_p()
+    assert lib.tde_workspace_create(3, 1024, ctypes.byref(ws)) == _capi.ENRANKS
+    assert lib.tde_workspace_create(2, 1000, ctypes.byref(ws)) == _capi.ESHAPE
+    assert lib.tde_workspace_create(2, 1024, None) == _capi.EINVAL
+    assert lib.tde_workspace_destroy(None) == _capi.OK
+    assert lib.tde_workspace_slot(None, 0) is None
+
+
+# ---- torch layer: the reference's names and schemas (src/register.cpp:4-15, torch_dist_ext/__init__.py) ------
+
+def test_torch_schemas_match_reference():
+    import torch_dist_ext_amd as tde
+    s = str(torch.ops.torch_dist_ext.allreduce_rms_fusion.default._schema)
+    assert s == ("torch_dist_ext::allreduce_rms_fusion(SymInt rank, SymInt nranks, Tensor allreduce_in, Tensor residual_in, "
+                 "Tensor rms_gamma, Tensor residual_out, Tensor norm_out, float eps, Tensor workspace) -> ()")
+    s = str(torch.ops.torch_dist_ext.allreduce_rms.default._schema)
+    assert s == ("torch_dist_ext::allreduce_rms(SymInt rank, SymInt nranks, Tensor allreduce_in, Tensor residual_in, "
+                 "Tensor rms_gamma, float eps, Tensor workspace) -> (Tensor, Tensor)") or "int rank, int nranks" in s
+    assert "get_workspace(Tensor ref) -> Tensor" in str(torch.ops.torch_dist_ext.get_workspace.default._schema)
+    for name in ("CommWorkspace", "allreduce_rms_fusion_impl", "CommProcess", "setup_env", "get_workspace", "allreduce_rms"):
+        assert hasattr(tde, name), name
+    assert tde.allreduce_rms is torch.ops.torch_dist_ext.allreduce_rms
+    import inspect
+    assert list(inspect.signature(tde.setup_env).parameters) == ["rank", "world_size", "max_size_in_bytes", "group"]
+    assert inspect.signature(tde.setup_env).parameters["max_size_in_bytes"].default == 8192 * 16384
+
+
+def test_fake_tensor_shapes():
+    import torch_dist_ext_amd as tde
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    tde.world_size_ = 4
+    try:
+        with FakeTensorMode():
+            x = torch.empty((128, 1024), dtype=torch.bfloat16)
+            g = torch.empty((1024,), dtype=torch.bfloat16)
+            ws = torch.ops.torch_dist_ext.get_workspace(x)
+            assert ws.shape == ((4 * 3 + 5) * 8,) and ws.dtype == torch.uint8
+            n, r = torch.ops.torch_dist_ext.allreduce_rms(0, 4, x, x, g, 1e-6, ws)
+            assert n.shape == x.shape and r.shape == x.shape and n.dtype == x.dtype
+            q, s, r2, n2 = torch.ops.torch_dist_ext.allreduce_rms_quant(0, 4, x, x, g, 1e-6, ws, tde.QUANT_FP8_GROUP, False)
+            assert q.dtype == torch.float8_e4m3fn and s.shape == (128, 8) and n2.numel() == 0
+            q, s, r2, n2 = torch.ops.torch_dist_ext.allreduce_rms_quant(0, 4, x, x, g, 1e-6, ws, tde.QUANT_INT8_TOKEN, True)
+            assert q.dtype == torch.int8 and s.shape == (128,) and n2.shape == x.shape
+    finally:
+        tde.world_size_ = None
+
+
+def test_cpu_tensors_are_rejected_not_silently_computed():
+    import torch_dist_ext_amd as tde
+    x = torch.zeros((4, 256), dtype=torch.bfloat16)
+    g = torch.ones((256,), dtype=torch.bfloat16)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        tde.allreduce_rms_fusion_impl(0, 2, x, x, g, torch.empty_like(x), torch.empty_like(x), 1e-6,
+                                      torch.zeros(88, dtype=torch.uint8))

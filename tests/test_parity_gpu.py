@@ -16,7 +16,7 @@ def _case(name, parts, residual, gamma, eps, quant, **kw):
     print("case", name, tuple(parts.shape), residual.dtype, quant, kw, flush=True)
     want = eager.reduce_rms(parts, residual, gamma, eps, quant)
     got = run_hip(parts, residual, gamma, eps, quant, **kw)
-    stats = check_against_oracle(got, want, quant)
+    stats = check_against_oracle(got, want, quant, gamma=gamma, eps=eps)
     print("  stats", stats, flush=True)
     return got, want, stats
 
@@ -70,3 +70,124 @@ def test_pointer_table_equals_direct(cuda_device):
     b = run_hip(p, r, g, 1e-5, "fp8_token", use_table=True, rank=3)
     for k in a:
         assert bits_equal(a[k], b[k]), k
+
+
+# Shapes of the reference's own tests: tokens {128,129} x 1024 x N=4 in fp32/bf16/fp16
+# (test/test_all_reduce_fusion.py:78-87) and the fp32 grid of test/unit_test.cpp:322-323, whose
+# hidden sizes 508 and 124 leave the last wavefront partly empty.
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tokens", [128, 129])
+def test_reference_python_test_shapes(cuda_device, dtype, tokens):
+    g = torch.Generator().manual_seed(tokens)
+    parts = torch.randn((4, tokens, 1024), generator=g).to(dtype)
+    residual = torch.randn((tokens, 1024), generator=g).to(dtype)
+    gamma = torch.randn((1024,), generator=g).to(dtype)  # the reference draws gamma from N(0,1)
+    _case("pytest-shape", parts, residual, gamma, 1e-6, "none")
+
+
+@pytest.mark.parametrize("hidden", [1024, 508, 124])
+@pytest.mark.parametrize("tokens", [513, 127, 3])
+def test_reference_unit_test_shapes_fp32(cuda_device, tokens, hidden):
+    g = torch.Generator().manual_seed(tokens * 7 + hidden)
+    parts = torch.rand((8, tokens, hidden), generator=g)
+    residual = torch.rand((tokens, hidden), generator=g)
+    gamma = torch.rand((hidden,), generator=g)
+    _case("unit-shape", parts, residual, gamma, 1e-6, "none")
+
+
+# ---- edge cases -----------------------------------------------------------------------------------------
+
+def test_empty_input_is_a_no_op(cuda_device):
+    p, r, g = eager.make_inputs(2, 0, 1024, torch.bfloat16, 1.0, seed=1)
+    got = run_hip(p, r, g, 1e-6, "fp8_token")
+    assert got["residual_out"].shape == (0, 1024) and got["q"].numel() == 0
+
+
+@pytest.mark.parametrize("hidden", [8, 64, 1016, 8192])
+@pytest.mark.parametrize("quant", ["none", "int8_token"])
+def test_ragged_and_extreme_hidden(cuda_device, hidden, quant):
+    p, r, g = eager.make_inputs(2, 5, hidden, torch.bfloat16, 1.0, seed=hidden)
+    _case("hidden", p, r, g, 1e-6, quant)
+
+
+def test_all_zero_rows_and_signed_zero(cuda_device):
+    p, r, g = eager.make_inputs(4, 6, 512, torch.bfloat16, 1.0, seed=2)
+    p[:, 1] = 0.0
+    r[1] = 0.0
+    p[:, 3] = -0.0
+    r[3] = -0.0
+    for quant in ("none", "fp8_token", "fp8_group", "int8_token"):
+        got, want, _ = _case("zeros", p, r, g, 1e-6, quant)
+        assert torch.all(got["residual_out"][3].view(torch.int16) == 0)   # -0 partials sum to +0
+        if quant != "none":
+            assert torch.all(got["scale"].reshape(6, -1)[1] == 0) and torch.all(got["q"][1].float() == 0)
+
+
+def test_rank_order_vector_on_gpu(cuda_device):
+    vals = [2.0 ** 24, 1.0, -(2.0 ** 24), 1.0]
+    parts = torch.tensor(vals, dtype=torch.bfloat16).view(4, 1, 1).expand(4, 3, 256).contiguous()
+    r = torch.zeros((3, 256), dtype=torch.bfloat16)
+    g = torch.ones((256,), dtype=torch.bfloat16)
+    got = run_hip(parts, r, g, 1e-6, "none")
+    assert torch.all(got["residual_out"].float() == 1.0)
+
+
+def test_sum_of_ones_row_reduction_all_wave_counts(cuda_device):
+    # mean(x^2) of a row of ones is exactly 1 for every hidden: checks the 64-lane + LDS reduction tree
+    for hidden in (8, 64, 1016, 1024, 5120, 7168, 8192):
+        parts = torch.zeros((2, 3, hidden), dtype=torch.bfloat16)
+        r = torch.ones((3, hidden), dtype=torch.bfloat16)
+        g = torch.ones((hidden,), dtype=torch.bfloat16)
+        got = run_hip(parts, r, g, 0.0, "none")
+        assert torch.all(got["norm_out"].float() == 1.0), hidden
+
+
+@pytest.mark.parametrize("vpt", [1, 2, 4])
+@pytest.mark.parametrize("prefetch,grid", [(1, 0), (2, 3)])
+def test_every_launch_geometry_agrees(cuda_device, vpt, prefetch, grid):
+    if prefetch == 2 and vpt != 1:
+        pytest.skip("the software-pipelined kernel exists for one vector per thread")
+    p, r, g = eager.make_inputs(8, 41, 8192, torch.bfloat16, 0.5, seed=77)
+    base = run_hip(p, r, g, 1e-5, "fp8_token")
+    _capi.tune_override(vpt, 0, grid, prefetch)
+    try:
+        other = run_hip(p, r, g, 1e-5, "fp8_token")
+    finally:
+        _capi.tune_override(0, 0, 0, 0)
+    want = eager.reduce_rms(p, r, g, 1e-5, "fp8_token")
+    check_against_oracle(other, want, "fp8_token", gamma=g, eps=1e-5)
+    assert bits_equal(base["residual_out"], other["residual_out"])
+
+
+def test_full_size_c3_properties(cuda_device):
+    """BASELINE c3 at full size on the device only (the CPU oracle is not run at this size here):
+    size-independent properties of the outputs."""
+    dev = cuda_device
+    gen = torch.Generator(device=dev).manual_seed(3)
+    N, T, H = 8, 2048, 8192
+    parts = [(torch.randn((T, H), generator=gen, device=dev) * 0.5).to(torch.bfloat16) for _ in range(N)]
+    res = torch.randn((T, H), generator=gen, device=dev).to(torch.bfloat16)
+    gamma = (torch.rand((H,), generator=gen, device=dev) + 0.5).to(torch.bfloat16)
+    import torch_dist_ext_amd as tde
+    out = tde.reduce_rms(parts, res, gamma, 1e-5, tde.QUANT_FP8_TOKEN, write_norm=True)
+    torch.cuda.synchronize()
+    # residual: the same fp32 rank-order sum written with torch ops on the device
+    acc = torch.zeros((T, H), device=dev)
+    for p in parts:
+        acc = acc + p.float()
+    x = (acc.to(torch.bfloat16).float() + res.float()).to(torch.bfloat16)
+    assert torch.equal(out["residual_out"].view(torch.int16), x.view(torch.int16))
+    y = out["norm_out"].float()
+    assert torch.equal(out["scale"], y.abs().amax(-1) / 448.0)                   # scale is amax/448 of the written rows
+    q = out["q"].float()
+    assert torch.all(q.abs().amax(-1) == 448.0)                                   # top code reached in every row
+    rms = torch.sqrt((y / gamma.float()).pow(2).mean(-1))
+    assert torch.all((rms - 1).abs() < 0.02)                                      # rows are normalized
+    # idempotence of the epilogue: re-quantizing the dequantized row with the same scale gives the same codes
+    deq = q * out["scale"].view(-1, 1)
+    q2 = (deq / out["scale"].view(-1, 1)).clamp(-448, 448).to(torch.float8_e4m3fn)
+    assert torch.equal(q2.view(torch.uint8), out["q"].view(torch.uint8))
+    # linearity of the reduce: permuting identical partial values among ranks that hold equal data changes nothing
+    out2 = tde.reduce_rms(parts, res, gamma, 1e-5, tde.QUANT_FP8_TOKEN, write_norm=True)
+    for k in out:
+        assert torch.equal(out[k].view(torch.uint8), out2[k].view(torch.uint8)), k         # deterministic run to run

@@ -1,0 +1,95 @@
+"""GPU: the reference's own call sequence (test/test_all_reduce_fusion.py:40-61) on one GPU:
+setup_env -> get_workspace -> allreduce_rms, with the peers' partials placed into the workspace slots."""
+import pytest
+import torch
+
+from oracle import eager
+
+from helpers import bits_equal, check_against_oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tde(cuda_device):
+    import torch_dist_ext_amd as m
+    return m
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tokens", [129, 128])
+def test_reference_call_sequence(tde, cuda_device, dtype, tokens):
+    world_size, hidden, eps, rank = 4, 1024, 1e-6, 1
+    print("case call-sequence", dtype, tokens, flush=True)
+    g = torch.Generator().manual_seed(tokens)
+    allreduce_in = torch.randn((world_size, tokens, hidden), generator=g).to(dtype)
+    residual_in = torch.randn((tokens, hidden), generator=g).to(dtype)
+    gamma = torch.randn((hidden,), generator=g).to(dtype)
+    want = eager.reduce_rms(allreduce_in, residual_in, gamma, eps)
+
+    tde.setup_env(rank, world_size)
+    local_in = allreduce_in[rank].to(cuda_device)
+    for r in range(world_size):
+        if r != rank:
+            tde.set_peer_partial(r, allreduce_in[r].to(cuda_device))
+    workspace = tde.get_workspace(local_in)
+    assert workspace.dtype == torch.uint8 and workspace.numel() == (3 * world_size + 5) * 8 and workspace.is_cuda
+    norm_out, residual_out = tde.allreduce_rms(rank, world_size, local_in, residual_in.to(cuda_device),
+                                               gamma.to(cuda_device), eps, workspace)
+    torch.cuda.synchronize()
+    got = {"norm_out": norm_out.cpu(), "residual_out": residual_out.cpu()}
+    print("  stats", check_against_oracle(got, want, "none", gamma=gamma, eps=eps), flush=True)
+
+
+@pytest.mark.parametrize("mode,quant", [(1, "fp8_token"), (2, "fp8_group"), (3, "int8_token")])
+def test_quant_op_through_workspace(tde, cuda_device, mode, quant):
+    world_size, tokens, hidden, eps, rank = 8, 70, 4096, 1e-5, 5
+    print("case quant-op", quant, flush=True)
+    p, r, g = eager.make_inputs(world_size, tokens, hidden, torch.bfloat16, 0.5, seed=31)
+    want = eager.reduce_rms(p, r, g, eps, quant)
+    tde.setup_env(rank, world_size, max_size_in_bytes=tokens * hidden * 2)
+    for k in range(world_size):
+        if k != rank:
+            tde.peer_partial(k, p[k].to(cuda_device)).copy_(p[k].to(cuda_device))
+    ws = tde.get_workspace(p[rank].to(cuda_device))
+    q, s, res_out, norm = torch.ops.torch_dist_ext.allreduce_rms_quant(
+        rank, world_size, p[rank].to(cuda_device), r.to(cuda_device), g.to(cuda_device), eps, ws, mode, True)
+    torch.cuda.synchronize()
+    got = {"q": q.cpu(), "scale": s.cpu(), "residual_out": res_out.cpu(), "norm_out": norm.cpu()}
+    print("  stats", check_against_oracle(got, want, quant, gamma=g, eps=eps), flush=True)
+    q2, s2, res2, norm2 = torch.ops.torch_dist_ext.allreduce_rms_quant(
+        rank, world_size, p[rank].to(cuda_device), r.to(cuda_device), g.to(cuda_device), eps, ws, mode, False)
+    assert norm2.numel() == 0 and bits_equal(q2.cpu(), got["q"]) and bits_equal(s2.cpu(), got["scale"])
+
+
+def test_local_list_op_and_staged(tde, cuda_device):
+    p, r, g = eager.make_inputs(4, 50, 2048, torch.float16, 1.0, seed=32)
+    want = eager.reduce_rms(p, r, g, 1e-6, "int8_token")
+    parts = [p[i].to(cuda_device) for i in range(4)]
+    a = tde.reduce_rms(parts, r.to(cuda_device), g.to(cuda_device), 1e-6, tde.QUANT_INT8_TOKEN, write_norm=True)
+    b = tde.reduce_rms(parts, r.to(cuda_device), g.to(cuda_device), 1e-6, tde.QUANT_INT8_TOKEN, write_norm=True,
+                       algo=tde.ALGO_STAGED)
+    torch.cuda.synchronize()
+    got = {k: v.cpu() for k, v in a.items()}
+    check_against_oracle(got, want, "int8_token", gamma=g, eps=1e-6)
+    for k in a:
+        assert bits_equal(a[k].cpu(), b[k].cpu()), k
+
+
+def test_error_paths_raise(tde, cuda_device):
+    x = torch.zeros((4, 256), dtype=torch.bfloat16, device=cuda_device)
+    g = torch.ones((256,), dtype=torch.bfloat16, device=cuda_device)
+    tde.setup_env(0, 2, max_size_in_bytes=4096)
+    ws = tde.get_workspace(x)
+    with pytest.raises(RuntimeError, match="nranks must be 2, 4 or 8"):
+        tde.allreduce_rms_fusion_impl(0, 3, x, x, g, torch.empty_like(x), torch.empty_like(x), 1e-6,
+                                      torch.zeros(200, dtype=torch.uint8, device=cuda_device))
+    with pytest.raises(RuntimeError, match="dtype"):
+        tde.allreduce_rms_fusion_impl(0, 2, x, x.float(), g, torch.empty_like(x), torch.empty_like(x), 1e-6, ws)
+    with pytest.raises(RuntimeError, match="exceed the slot size"):
+        tde.peer_partial(1, torch.zeros((64, 256), dtype=torch.bfloat16, device=cuda_device))
+    with pytest.raises(RuntimeError, match="rank"):
+        tde.CommWorkspace(5, 4, 256, 4096)
+    y = torch.zeros((4, 8200), dtype=torch.bfloat16, device=cuda_device)
+    with pytest.raises(AssertionError):
+        tde.allreduce_rms(0, 2, y, y, torch.ones(8200, dtype=torch.bfloat16, device=cuda_device), 1e-6, ws)

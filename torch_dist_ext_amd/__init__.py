@@ -25,7 +25,7 @@ this_dir = os.path.dirname(os.path.abspath(__file__))
 filename = os.path.join(this_dir, "libtorch_dist_ext.so")
 if not (os.path.exists(filename) and os.path.exists(_capi.LIB_PATH)):
     raise ImportError(
-        "torch_dist_ext_amd: %s / %s not built. Run `python -m torch_dist_ext_amd._build` "
+        "torch_dist_ext_amd: %s / %s not built. Run `python torch_dist_ext_amd/_build.py` "
         "(there is no CPU fallback)." % (os.path.basename(filename), os.path.basename(_capi.LIB_PATH)))
 _capi.load()  # libtde_hip.so first, so the extension resolves against the in-tree copy
 torch.ops.load_library(filename)

@@ -5,7 +5,8 @@
                          libtde_hip.so (the name the reference's package loads, torch_dist_ext/__init__.py:8-12)
 
 Both land next to this file so they travel with the source tree.
-Run as `python -m torch_dist_ext_amd._build`.
+Run as `python torch_dist_ext_amd/_build.py` (by path: importing the package needs the libraries
+this script produces).
 """
 import os
 import subprocess

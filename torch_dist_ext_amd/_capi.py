@@ -17,7 +17,7 @@ ALGO_AUTO, ALGO_FUSED, ALGO_STAGED = 0, 1, 2
 
 # Every symbol include/tde_abi.h declares.
 EXPORTS = (
-    "tde_abi_version", "tde_status_string", "tde_last_hip_error", "tde_plan", "tde_reduce_rms", "tde_tune_override",
+    "tde_abi_version", "tde_status_string", "tde_last_hip_error", "tde_plan", "tde_reduce_rms", "tde_tune_override", "tde_probe_copy",
     "tde_workspace_create", "tde_workspace_destroy", "tde_workspace_slot", "tde_workspace_stage",
     "tde_workspace_slot_bytes", "tde_workspace_nranks", "tde_workspace_fill_table",
 )
@@ -63,7 +63,7 @@ def load():
     if _lib is not None:
         return _lib
     if not os.path.exists(LIB_PATH):
-        raise ImportError("%s not built; run `python -m torch_dist_ext_amd._build`" % LIB_PATH)
+        raise ImportError("%s not built; run `python torch_dist_ext_amd/_build.py`" % LIB_PATH)
     lib = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
     lib.tde_abi_version.restype = ctypes.c_int
     lib.tde_status_string.restype = ctypes.c_char_p
@@ -74,7 +74,9 @@ def load():
     lib.tde_reduce_rms.restype = ctypes.c_int
     lib.tde_reduce_rms.argtypes = [ctypes.POINTER(Problem), ctypes.POINTER(Buffers), ctypes.c_void_p]
     lib.tde_tune_override.restype = ctypes.c_int
-    lib.tde_tune_override.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
+    lib.tde_tune_override.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
+    lib.tde_probe_copy.restype = ctypes.c_int
+    lib.tde_probe_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
     lib.tde_workspace_create.restype = ctypes.c_int
     lib.tde_workspace_create.argtypes = [ctypes.c_int32, ctypes.c_int64, ctypes.POINTER(ctypes.c_void_p)]
     lib.tde_workspace_destroy.restype = ctypes.c_int
@@ -130,5 +132,9 @@ def reduce_rms(problem, partials, residual_in, residual_out, gamma, norm_out=Non
     check(load().tde_reduce_rms(ctypes.byref(problem), ctypes.byref(b), stream))
 
 
-def tune_override(vecs_per_thread=0, rows_per_block=0, max_grid=0):
-    check(load().tde_tune_override(vecs_per_thread, rows_per_block, max_grid))
+def tune_override(vecs_per_thread=0, rows_per_block=0, max_grid=0, prefetch=0):
+    check(load().tde_tune_override(vecs_per_thread, rows_per_block, max_grid, prefetch))
+
+
+def probe_copy(dst, src, nbytes, stream=None):
+    check(load().tde_probe_copy(dst, src, nbytes, stream))

@@ -83,7 +83,8 @@ struct ElemF16 {
     static __device__ __forceinline__ void unpack(u32x4 raw, float (&f)[VEC]) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            f16x2 h = __builtin_bit_cast(f16x2, raw[i]);
+            const uint32_t w = raw[i]; // copy first: bit_cast applied straight to a vector element reads lane 0
+            const f16x2 h = __builtin_bit_cast(f16x2, w);
             f[2 * i] = (float)h[0];
             f[2 * i + 1] = (float)h[1];
         }
@@ -104,7 +105,10 @@ struct ElemF32 {
     static constexpr int BYTES = 4;
     static __device__ __forceinline__ void unpack(u32x4 raw, float (&f)[VEC]) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) f[i] = __builtin_bit_cast(float, raw[i]);
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t w = raw[i]; // copy first: bit_cast applied straight to a vector element reads lane 0
+            f[i] = __builtin_bit_cast(float, w);
+        }
     }
     static __device__ __forceinline__ u32x4 pack(const float (&f)[VEC]) {
         u32x4 raw;
@@ -169,22 +173,32 @@ __device__ __forceinline__ float row_reduce(float v, float *slots, int wave, int
 
 // Streaming (non-temporal) 128-bit access at a wavefront-uniform base plus a 32-bit lane offset:
 // the form that maps to global_load/store_dwordx4 with an SGPR base.
-// Every buffer is device (global) memory, so the accesses are typed as address space 1 and never
+// Every buffer is device (global) memory, so plain accesses are typed as address space 1 and never
 // go through the flat aperture check.
 #define TDE_GLOBAL __attribute__((address_space(1)))
 template <class V>
 __device__ __forceinline__ const TDE_GLOBAL V *global_ptr(const void *base, uint32_t byte_off) {
     return (const TDE_GLOBAL V *)((const TDE_GLOBAL char *)base + byte_off);
 }
-template <class V>
-__device__ __forceinline__ TDE_GLOBAL V *global_ptr(void *base, uint32_t byte_off) {
-    return (TDE_GLOBAL V *)((TDE_GLOBAL char *)base + byte_off);
+
+// Row-sized buffer resources.  A row is addressed as (wavefront-uniform 128-bit resource in SGPRs)
+// + (32-bit lane offset in one VGPR).  The resource's size is the row's byte length, or 0 for a row
+// past the end: the hardware then returns zeros for loads and drops stores, so neither partially
+// filled wavefronts nor tail rows need a branch.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr int kRsrcFlags = 0x00020000; // raw buffer, 32-bit data format (gfx9 family encoding)
+constexpr int kAuxStream = 2;          // nt: streamed once, do not keep in cache
+constexpr int kAuxDefault = 0;
+
+__device__ __forceinline__ rsrc_t row_rsrc(const void *base, int64_t byte_off, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc((void *)(static_cast<const char *>(base) + byte_off), 0, (int)bytes,
+                                             kRsrcFlags);
 }
-__device__ __forceinline__ u32x4 load_stream(const void *base, uint32_t byte_off) {
-    return __builtin_nontemporal_load(global_ptr<u32x4>(base, byte_off));
+__device__ __forceinline__ u32x4 rsrc_load16(rsrc_t r, uint32_t off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, kAuxStream);
 }
-__device__ __forceinline__ void store_stream(void *base, uint32_t byte_off, u32x4 v) {
-    __builtin_nontemporal_store(v, global_ptr<u32x4>(base, byte_off));
+__device__ __forceinline__ void rsrc_store16(rsrc_t r, uint32_t off, u32x4 v) {
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)off, 0, kAuxStream);
 }
 
 // Pack VEC fp32 values (already clamped to +-448) to OCP e4m3 bytes, round to nearest even.
@@ -213,19 +227,40 @@ __device__ __forceinline__ void pack_int8(const float (&q)[VEC], uint32_t (&out)
     }
 }
 
+// y / d, correctly rounded, for a divisor shared by many elements.  `rcp` must be the correctly
+// rounded 1/d.  q0 = RN(y*rcp) is within one ulp of the quotient; the residual y - q0*d is exact
+// in one fma; adding residual*rcp back in a second fma rounds to the correctly rounded quotient
+// (Markstein's division theorem) as long as nothing underflows.  Callers take this path only when
+// d is far from the subnormal and overflow ranges and use a plain division otherwise.
+__device__ __forceinline__ float div_shared(float y, float d, float rcp) {
+    const float q0 = y * rcp;
+    const float e = __builtin_fmaf(-q0, d, y);
+    return __builtin_fmaf(e, rcp, q0);
+}
+
+// The loads of one row: N partial vectors and one residual vector per owned 16-byte column slot.
+template <int NP, int VPT>
+struct RowLoads {
+    u32x4 p[VPT][NP];
+    u32x4 r[VPT];
+};
+
 // ---------------------------------------------------------------------------------------------
 // The row kernel.
 //   E      element traits
 //   N      number of partials summed per element; N == 0 means "the sum was staged":
 //          part[0] already holds s (a T-typed [tokens,hidden] buffer)
-//   VPT    16-byte vectors per thread per row
+//   VPT    16-byte vectors per thread per row (1 or 2)
 //   Q      tde_quant
 //   WN     write the T-typed normed row (always true for Q == NONE)
+//   PF     software pipeline: the loads of the block's next row are issued before the current row is
+//          consumed, so a workgroup always has a full row of requests in flight
 // Block layout: rows_per_block row groups of threads_per_row threads; thread t of a row group
 // owns vectors t, t + threads_per_row, ... (coalesced 1 KiB per wavefront per load).
 // ---------------------------------------------------------------------------------------------
-template <class E, int N, int VPT, int Q, bool WN>
-__global__ void __launch_bounds__(1024 / VPT) row_kernel(const RowArgs a) {
+template <class E, int N, int VPT, int Q, bool WN, bool PF>
+__global__ void __launch_bounds__(1024 / VPT)
+    __attribute__((amdgpu_waves_per_eu(PF ? 4 : (VPT == 1 ? 8 : (VPT == 2 ? 6 : 2))))) row_kernel(const RowArgs a) {
     constexpr int VEC = E::VEC;
     constexpr int NP = (N == 0) ? 1 : N;
     __shared__ float lds_sum[2][kMaxWavesPerBlock];
@@ -239,6 +274,7 @@ __global__ void __launch_bounds__(1024 / VPT) row_kernel(const RowArgs a) {
     const int group = __builtin_amdgcn_readfirstlane(tid / tpr); // uniform inside a wavefront
     const int t = tid - group * tpr;
     const int first_wave = group * waves_per_row;
+    const uint32_t row_bytes = (uint32_t)a.hidden * E::BYTES;
 
     const void *part[NP];
 #pragma unroll
@@ -249,48 +285,56 @@ __global__ void __launch_bounds__(1024 / VPT) row_kernel(const RowArgs a) {
 
     // gamma is shared by every row this block touches: keep it in registers.
     u32x4 gamma_raw[VPT];
-    bool col_ok[VPT];
     uint32_t lane_off[VPT]; // byte offset of this thread's vector j inside a row
 #pragma unroll
     for (int j = 0; j < VPT; ++j) {
         const int v = j * tpr + t;
-        col_ok[j] = v < a.nvec;
         lane_off[j] = (uint32_t)v * 16u;
-        gamma_raw[j] = col_ok[j] ? *global_ptr<u32x4>(a.gamma, lane_off[j]) : u32x4{0, 0, 0, 0};
+        gamma_raw[j] = (v < a.nvec) ? *global_ptr<u32x4>(a.gamma, lane_off[j]) : u32x4{0, 0, 0, 0};
     }
 
+    auto issue_loads = [&](RowLoads<NP, VPT> &d, int64_t row) {
+        const uint32_t bytes = (row < a.tokens) ? row_bytes : 0u;
+        const int64_t row_byte = row * (int64_t)row_bytes;
+#pragma unroll
+        for (int r = 0; r < NP; ++r) {
+            const rsrc_t rs = row_rsrc(part[r], row_byte, bytes);
+#pragma unroll
+            for (int j = 0; j < VPT; ++j) d.p[j][r] = rsrc_load16(rs, lane_off[j]);
+        }
+        const rsrc_t rr = row_rsrc(a.residual_in, row_byte, bytes);
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) d.r[j] = rsrc_load16(rr, lane_off[j]);
+    };
+
     const int64_t row_stride = (int64_t)gridDim.x * a.rows_per_block;
+    int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block;
+    RowLoads<NP, VPT> cur;
+    if constexpr (PF) issue_loads(cur, row0 + group);
+
     int parity = 0;
-    for (int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block; row0 < a.tokens; row0 += row_stride, parity ^= 1) {
+    for (; row0 < a.tokens; row0 += row_stride, parity ^= 1) {
         const int64_t row = row0 + group;
         const bool row_ok = row < a.tokens;
-        const int64_t row_elem = row * (int64_t)a.hidden;
-        const int64_t row_byte = row_elem * E::BYTES; // wavefront-uniform
+        const uint32_t bytes = row_ok ? row_bytes : 0u;
+        const int64_t row_byte = row * (int64_t)row_bytes; // wavefront-uniform
 
-        // ---- issue every load of the row before consuming any ---------------------------------
-        u32x4 praw[VPT][NP];
-        u32x4 rraw[VPT];
-#pragma unroll
-        for (int j = 0; j < VPT; ++j) {
-#pragma unroll
-            for (int r = 0; r < NP; ++r) praw[j][r] = u32x4{0, 0, 0, 0};
-            rraw[j] = u32x4{0, 0, 0, 0};
-            if (row_ok && col_ok[j]) {
-#pragma unroll
-                for (int r = 0; r < NP; ++r)
-                    praw[j][r] = load_stream(static_cast<const char *>(part[r]) + row_byte, lane_off[j]);
-                rraw[j] = load_stream(static_cast<const char *>(a.residual_in) + row_byte, lane_off[j]);
-            }
+        RowLoads<NP, VPT> nxt;
+        if constexpr (PF) {
+            issue_loads(nxt, row + row_stride); // past-the-end rows load nothing
+        } else {
+            issue_loads(cur, row);
         }
 
         // ---- reduce, residual add, sum of squares ------------------------------------------------
+        const rsrc_t res_out = row_rsrc(a.residual_out, row_byte, bytes);
         u32x4 xraw[VPT];
         float sumsq = 0.0f;
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
             float s[VEC];
             if constexpr (N == 0) {
-                E::unpack(praw[j][0], s);
+                E::unpack(cur.p[j][0], s);
             } else {
                 float acc[VEC];
 #pragma unroll
@@ -298,22 +342,25 @@ __global__ void __launch_bounds__(1024 / VPT) row_kernel(const RowArgs a) {
 #pragma unroll
                 for (int r = 0; r < NP; ++r) {
                     float p[VEC];
-                    E::unpack(praw[j][r], p);
+                    E::unpack(cur.p[j][r], p);
 #pragma unroll
                     for (int i = 0; i < VEC; ++i) acc[i] += p[i];
                 }
                 E::unpack(E::pack(acc), s);
             }
             float res[VEC], x[VEC];
-            E::unpack(rraw[j], res);
+            E::unpack(cur.r[j], res);
 #pragma unroll
             for (int i = 0; i < VEC; ++i) x[i] = s[i] + res[i];
             xraw[j] = E::pack(x);
-            const bool ok = row_ok && col_ok[j];
-            if (ok) store_stream(static_cast<char *>(a.residual_out) + row_byte, lane_off[j], xraw[j]);
+            rsrc_store16(res_out, lane_off[j], xraw[j]);
             E::unpack(xraw[j], x);
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) sumsq += x[i] * x[i];
+            for (int i = 0; i < VEC; ++i) {
+                // 2-byte types: x*x is exact in fp32, so the fused form rounds exactly like mul-then-add.
+                if constexpr (E::BYTES == 2) sumsq = __builtin_fmaf(x[i], x[i], sumsq);
+                else sumsq += x[i] * x[i];
+            }
         }
         sumsq = row_reduce<OpSum>(sumsq, lds_sum[parity], wave, lane, first_wave, waves_per_row);
         const float rs = 1.0f / __builtin_sqrtf(sumsq / a.hidden_f + a.eps);
@@ -332,9 +379,9 @@ __global__ void __launch_bounds__(1024 / VPT) row_kernel(const RowArgs a) {
 #pragma unroll
             for (int i = 0; i < VEC; ++i) y[i] = g[i] * y[i];
             yraw[j] = E::pack(y);
-            const bool ok = row_ok && col_ok[j];
             if constexpr (Q == TDE_QUANT_NONE || WN) {
-                if (ok) store_stream(static_cast<char *>(a.norm_out) + row_byte, lane_off[j], yraw[j]);
+                const rsrc_t norm_out = row_rsrc(a.norm_out, row_byte, bytes);
+                rsrc_store16(norm_out, lane_off[j], yraw[j]);
             }
             if constexpr (Q != TDE_QUANT_NONE) {
                 E::unpack(yraw[j], y);
@@ -351,16 +398,16 @@ __global__ void __launch_bounds__(1024 / VPT) row_kernel(const RowArgs a) {
             float scale[VPT];
             if constexpr (Q == TDE_QUANT_FP8_GROUP) {
                 constexpr int LANES_PER_GROUP = TDE_QUANT_GROUP / VEC; // 16 (2-byte types) or 32 (fp32)
+                const int64_t groups_per_row = a.hidden / TDE_QUANT_GROUP;
+                const rsrc_t sc_out = row_rsrc(a.scale_out, row * groups_per_row * 4, row_ok ? (uint32_t)groups_per_row * 4u : 0u);
 #pragma unroll
                 for (int j = 0; j < VPT; ++j) {
                     float m = row16_reduce<OpMax>(amax[j]);
                     if constexpr (LANES_PER_GROUP == 32) m = fmaxf(m, __shfl_xor(m, 16, kWave));
                     scale[j] = m / QMAX;
-                    const int v = j * tpr + t;
-                    if (row_ok && col_ok[j] && (lane & (LANES_PER_GROUP - 1)) == 0) {
-                        const int64_t groups_per_row = a.hidden / TDE_QUANT_GROUP;
-                        ((TDE_GLOBAL float *)a.scale_out)[row * groups_per_row + v / LANES_PER_GROUP] = scale[j];
-                    }
+                    if ((lane & (LANES_PER_GROUP - 1)) == 0)
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, scale[j]), sc_out,
+                                                              (int)((lane_off[j] / 16u / LANES_PER_GROUP) * 4u), 0, kAuxDefault);
                 }
             } else {
                 float m = amax[0];
@@ -372,30 +419,37 @@ __global__ void __launch_bounds__(1024 / VPT) row_kernel(const RowArgs a) {
                 for (int j = 0; j < VPT; ++j) scale[j] = sc;
                 if (row_ok && t == 0) ((TDE_GLOBAL float *)a.scale_out)[row] = sc;
             }
+            const rsrc_t q_out = row_rsrc(a.q_out, row * (int64_t)a.hidden, row_ok ? (uint32_t)a.hidden : 0u);
 #pragma unroll
             for (int j = 0; j < VPT; ++j) {
                 float y[VEC], q[VEC];
                 E::unpack(yraw[j], y);
                 const float div = (scale[j] > 0.0f) ? scale[j] : 1.0f;
+                const float rcp = 1.0f / div;
+                // One wavefront-uniform decision, so the common path carries no per-lane branch.
+                const bool unsafe = !(div > 0x1p-60f && div < 0x1p60f);
+                if (__builtin_amdgcn_ballot_w64(unsafe) == 0) {
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) q[i] = fminf(fmaxf(y[i] / div, -QMAX), QMAX);
+                    for (int i = 0; i < VEC; ++i) q[i] = fminf(fmaxf(div_shared(y[i], div, rcp), -QMAX), QMAX);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) q[i] = fminf(fmaxf(y[i] / div, -QMAX), QMAX);
+                }
                 uint32_t codes[VEC / 4];
                 if constexpr (Q == TDE_QUANT_INT8_TOKEN)
                     pack_int8<VEC>(q, codes);
                 else
                     pack_fp8<VEC>(q, codes);
-                if (row_ok && col_ok[j]) {
-                    char *dst = static_cast<char *>(a.q_out) + row_elem;
-                    const uint32_t code_off = (lane_off[j] / 16u) * (uint32_t)VEC;
-                    if constexpr (VEC == 8) {
-                        u32x2 w = {codes[0], codes[1]};
-                        __builtin_nontemporal_store(w, global_ptr<u32x2>(dst, code_off));
-                    } else {
-                        __builtin_nontemporal_store(codes[0], global_ptr<uint32_t>(dst, code_off));
-                    }
+                const uint32_t code_off = (lane_off[j] / 16u) * (uint32_t)VEC;
+                if constexpr (VEC == 8) {
+                    u32x2 w = {codes[0], codes[1]};
+                    __builtin_amdgcn_raw_buffer_store_b64(w, q_out, (int)code_off, 0, kAuxStream);
+                } else {
+                    __builtin_amdgcn_raw_buffer_store_b32(codes[0], q_out, (int)code_off, 0, kAuxStream);
                 }
             }
         }
+        if constexpr (PF) cur = nxt;
     }
 }
 
@@ -441,6 +495,7 @@ struct Geometry {
     int rows_per_block;
     int block_threads;
     int64_t grid;
+    bool prefetch;
 };
 
 // Per-dtype launchers, defined in tde_rows_<dtype>.hip.
@@ -452,11 +507,11 @@ hipError_t launch_reduce_f16(int n, const RowArgs &a, int64_t total_vecs, hipStr
 hipError_t launch_reduce_f32(int n, const RowArgs &a, int64_t total_vecs, hipStream_t s);
 
 // Instantiation + dispatch body used by the three per-dtype translation units.
-template <class E, int N, int VPT>
-hipError_t launch_rows_nv(int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s) {
+template <class E, int N, int VPT, bool PF>
+hipError_t launch_rows_nvp(int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s) {
     const dim3 grid((unsigned)g.grid), block((unsigned)g.block_threads);
-#define TDE_LAUNCH(QM, WNB)                                                   \
-    hipLaunchKernelGGL((row_kernel<E, N, VPT, QM, WNB>), grid, block, 0, s, a); \
+#define TDE_LAUNCH(QM, WNB)                                                       \
+    hipLaunchKernelGGL((row_kernel<E, N, VPT, QM, WNB, PF>), grid, block, 0, s, a); \
     return hipGetLastError();
     switch (q) {
     case TDE_QUANT_NONE: TDE_LAUNCH(TDE_QUANT_NONE, true)
@@ -473,11 +528,9 @@ hipError_t launch_rows_nv(int q, bool wn, const RowArgs &a, const Geometry &g, h
 
 template <class E, int N>
 hipError_t launch_rows_n(int vpt, int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s) {
-    switch (vpt) {
-    case 1: return launch_rows_nv<E, N, 1>(q, wn, a, g, s);
-    case 2: return launch_rows_nv<E, N, 2>(q, wn, a, g, s);
-    case 4: return launch_rows_nv<E, N, 4>(q, wn, a, g, s);
-    }
+    if (vpt == 1) return g.prefetch ? launch_rows_nvp<E, N, 1, true>(q, wn, a, g, s) : launch_rows_nvp<E, N, 1, false>(q, wn, a, g, s);
+    if (vpt == 2) return launch_rows_nvp<E, N, 2, false>(q, wn, a, g, s);
+    if (vpt == 4) return launch_rows_nvp<E, N, 4, false>(q, wn, a, g, s);
     return hipErrorInvalidValue;
 }
 
