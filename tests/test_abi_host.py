@@ -113,9 +113,8 @@ def test_reduce_rms_argument_checks_need_no_gpu():
     prob.algo = _capi.ALGO_AUTO
     prob.quant = _capi.QUANT_FP8_TOKEN
     assert lib.tde_reduce_rms(ctypes.byref(prob), ctypes.byref(b), None) == _capi.EINVAL      # quant without q/scale
-    prob.quant = _capi.QUANT_NONE
     prob.tokens = 0
-    assert lib.tde_reduce_rms(ctypes.byref(prob), ctypes.byref(b), None) == _capi.OK          # empty input: no launch
+    assert lib.tde_reduce_rms(ctypes.byref(prob), ctypes.byref(_capi.Buffers()), None) == _capi.OK   # empty input: no launch
 
 
 def test_workspace_argument_checks_need_no_gpu():

@@ -177,17 +177,23 @@ def test_full_size_c3_properties(cuda_device):
         acc = acc + p.float()
     x = (acc.to(torch.bfloat16).float() + res.float()).to(torch.bfloat16)
     assert torch.equal(out["residual_out"].view(torch.int16), x.view(torch.int16))
-    y = out["norm_out"].float()
-    assert torch.equal(out["scale"], y.abs().amax(-1) / 448.0)                   # scale is amax/448 of the written rows
-    q = out["q"].float()
+    # the remaining checks run on the host: torch's device division by a Python scalar multiplies by
+    # a reciprocal and is not the IEEE quotient
+    y = out["norm_out"].float().cpu()
+    scale = out["scale"].cpu()
+    assert torch.equal(scale, y.abs().amax(-1) / 448.0)                           # scale is amax/448 of the written rows
+    q = out["q"].cpu().float()
     assert torch.all(q.abs().amax(-1) == 448.0)                                   # top code reached in every row
-    rms = torch.sqrt((y / gamma.float()).pow(2).mean(-1))
+    rms = torch.sqrt((y / gamma.float().cpu()).pow(2).mean(-1))
     assert torch.all((rms - 1).abs() < 0.02)                                      # rows are normalized
+    # the codes are the oracle's quantizer applied to the written rows, bit for bit
+    q_own, s_own = eager.quant_fp8(out["norm_out"].cpu(), None)
+    assert torch.equal(q_own.view(torch.uint8), out["q"].cpu().view(torch.uint8)) and torch.equal(s_own, scale)
     # idempotence of the epilogue: re-quantizing the dequantized row with the same scale gives the same codes
-    deq = q * out["scale"].view(-1, 1)
-    q2 = (deq / out["scale"].view(-1, 1)).clamp(-448, 448).to(torch.float8_e4m3fn)
-    assert torch.equal(q2.view(torch.uint8), out["q"].view(torch.uint8))
-    # linearity of the reduce: permuting identical partial values among ranks that hold equal data changes nothing
+    deq = q * scale.view(-1, 1)
+    q2 = (deq / scale.view(-1, 1)).clamp(-448, 448).to(torch.float8_e4m3fn)
+    assert torch.equal(q2.view(torch.uint8), out["q"].cpu().view(torch.uint8))
+    # determinism: a second launch on the same inputs writes the same bits
     out2 = tde.reduce_rms(parts, res, gamma, 1e-5, tde.QUANT_FP8_TOKEN, write_norm=True)
     for k in out:
         assert torch.equal(out[k].view(torch.uint8), out2[k].view(torch.uint8)), k         # deterministic run to run

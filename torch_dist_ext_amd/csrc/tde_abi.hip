@@ -190,6 +190,7 @@ int tde_reduce_rms(const tde_problem *p, const tde_buffers *b, void *hip_stream)
     const int st = validate(p, &g);
     if (st != TDE_OK) return st;
     if (b == nullptr) return TDE_EINVAL;
+    if (p->tokens == 0) return TDE_OK; // nothing to do; empty buffers may be null
     const bool quant = p->quant != TDE_QUANT_NONE;
     const bool wn = !quant || p->write_norm != 0;
     const bool staged = p->algo == TDE_ALGO_STAGED;
@@ -207,7 +208,6 @@ int tde_reduce_rms(const tde_problem *p, const tde_buffers *b, void *hip_stream)
         return TDE_EALIGN;
     if (quant && ((reinterpret_cast<uintptr_t>(b->q_out) & 7u) || (reinterpret_cast<uintptr_t>(b->scale_out) & 3u)))
         return TDE_EALIGN;
-    if (p->tokens == 0) return TDE_OK;
 
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     tde::RowArgs a{};
