@@ -57,9 +57,7 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
 
     // Vectors per thread: long rows use small workgroups that each keep many loads in flight
     // (measured best on MI355X: 256-thread groups with 4 vectors per thread at 1024 vectors per row).
-    int vpt = 1;
-    if (nvec >= 768) vpt = 4;
-    else if (nvec >= 384) vpt = 2;
+    int vpt = (nvec >= 768) ? 4 : 1;
     if (g_force_vpt == 1 || g_force_vpt == 2 || g_force_vpt == 4) vpt = g_force_vpt;
     const int64_t lanes = (nvec + vpt - 1) / vpt;
     const int tpr = (int)((lanes + 63) / 64 * 64);

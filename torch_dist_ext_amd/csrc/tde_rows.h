@@ -187,7 +187,11 @@ __device__ __forceinline__ const TDE_GLOBAL V *global_ptr(const void *base, uint
 // filled wavefronts nor tail rows need a branch.
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 constexpr int kRsrcFlags = 0x00020000; // raw buffer, 32-bit data format (gfx9 family encoding)
-constexpr int kAuxStream = 2;          // nt: streamed once, do not keep in cache
+constexpr int kAuxStream = 2;          // loads, nt: streamed once, do not keep in cache (7.0 vs 6.4 TB/s read ceiling)
+#ifndef TDE_AUX_STORE
+#define TDE_AUX_STORE 16
+#endif
+constexpr int kAuxStore = TDE_AUX_STORE; // stores, sc1: measured best for the mixed 6:1 read/write stream (nt stores cost ~8 %)
 constexpr int kAuxDefault = 0;
 
 __device__ __forceinline__ rsrc_t row_rsrc(const void *base, int64_t byte_off, uint32_t bytes) {
@@ -198,7 +202,7 @@ __device__ __forceinline__ u32x4 rsrc_load16(rsrc_t r, uint32_t off) {
     return __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, kAuxStream);
 }
 __device__ __forceinline__ void rsrc_store16(rsrc_t r, uint32_t off, u32x4 v) {
-    __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)off, 0, kAuxStream);
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)off, 0, kAuxStore);
 }
 
 // Pack VEC fp32 values (already clamped to +-448) to OCP e4m3 bytes, round to nearest even.
@@ -260,7 +264,7 @@ struct RowLoads {
 // ---------------------------------------------------------------------------------------------
 template <class E, int N, int VPT, int Q, bool WN, bool PF>
 __global__ void __launch_bounds__(1024 / VPT)
-    __attribute__((amdgpu_waves_per_eu(PF ? 4 : (VPT == 1 ? 8 : (VPT == 2 ? 6 : 2))))) row_kernel(const RowArgs a) {
+    __attribute__((amdgpu_waves_per_eu(PF ? 4 : (VPT == 1 ? 8 : (VPT == 2 ? 5 : 2))))) row_kernel(const RowArgs a) {
     constexpr int VEC = E::VEC;
     constexpr int NP = (N == 0) ? 1 : N;
     __shared__ float lds_sum[2][kMaxWavesPerBlock];
@@ -276,22 +280,22 @@ __global__ void __launch_bounds__(1024 / VPT)
     const int first_wave = group * waves_per_row;
     const uint32_t row_bytes = (uint32_t)a.hidden * E::BYTES;
 
+    // Partial pointers: from the argument block, or (one uniform branch, batched scalar loads)
+    // from the device pointer table for the entries the host left null.
     const void *part[NP];
 #pragma unroll
-    for (int r = 0; r < NP; ++r) {
-        part[r] = a.part[r];
-        if (part[r] == nullptr) part[r] = a.table[r];
+    for (int r = 0; r < NP; ++r) part[r] = a.part[r];
+    if (a.table != nullptr) {
+#pragma unroll
+        for (int r = 0; r < NP; ++r) {
+            const void *from_table = a.table[r];
+            part[r] = (part[r] != nullptr) ? part[r] : from_table;
+        }
     }
 
-    // gamma is shared by every row this block touches: keep it in registers.
-    u32x4 gamma_raw[VPT];
     uint32_t lane_off[VPT]; // byte offset of this thread's vector j inside a row
 #pragma unroll
-    for (int j = 0; j < VPT; ++j) {
-        const int v = j * tpr + t;
-        lane_off[j] = (uint32_t)v * 16u;
-        gamma_raw[j] = (v < a.nvec) ? *global_ptr<u32x4>(a.gamma, lane_off[j]) : u32x4{0, 0, 0, 0};
-    }
+    for (int j = 0; j < VPT; ++j) lane_off[j] = (uint32_t)(j * tpr + t) * 16u;
 
     auto issue_loads = [&](RowLoads<NP, VPT> &d, int64_t row) {
         const uint32_t bytes = (row < a.tokens) ? row_bytes : 0u;
@@ -309,8 +313,19 @@ __global__ void __launch_bounds__(1024 / VPT)
 
     const int64_t row_stride = (int64_t)gridDim.x * a.rows_per_block;
     int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block;
+
+    // The first row's loads go out before anything else touches memory; gamma (shared by every row,
+    // served from L2) is requested behind them and is only needed after the first row reduction.
     RowLoads<NP, VPT> cur;
-    if constexpr (PF) issue_loads(cur, row0 + group);
+    issue_loads(cur, row0 + group);
+    __builtin_amdgcn_sched_barrier(0);
+    u32x4 gamma_raw[VPT];
+    {
+        const rsrc_t gr = row_rsrc(a.gamma, 0, row_bytes);
+#pragma unroll
+        for (int j = 0; j < VPT; ++j)
+            gamma_raw[j] = __builtin_amdgcn_raw_buffer_load_b128(gr, (int)lane_off[j], 0, kAuxDefault);
+    }
 
     int parity = 0;
     for (; row0 < a.tokens; row0 += row_stride, parity ^= 1) {
@@ -320,11 +335,7 @@ __global__ void __launch_bounds__(1024 / VPT)
         const int64_t row_byte = row * (int64_t)row_bytes; // wavefront-uniform
 
         RowLoads<NP, VPT> nxt;
-        if constexpr (PF) {
-            issue_loads(nxt, row + row_stride); // past-the-end rows load nothing
-        } else {
-            issue_loads(cur, row);
-        }
+        if constexpr (PF) issue_loads(nxt, row + row_stride); // past-the-end rows load nothing
 
         // ---- reduce, residual add, sum of squares ------------------------------------------------
         const rsrc_t res_out = row_rsrc(a.residual_out, row_byte, bytes);
@@ -372,7 +383,9 @@ __global__ void __launch_bounds__(1024 / VPT)
         for (int j = 0; j < VPT; ++j) {
             float x[VEC], g[VEC], y[VEC];
             E::unpack(xraw[j], x);
-            E::unpack(gamma_raw[j], g);
+            u32x4 graw = gamma_raw[j];
+            asm volatile("" : "+v"(graw)); // unpack here, per row: hoisting it would put a wait for gamma before the row loads
+            E::unpack(graw, g);
 #pragma unroll
             for (int i = 0; i < VEC; ++i) y[i] = x[i] * rs;
             E::unpack(E::pack(y), y);
@@ -443,13 +456,17 @@ __global__ void __launch_bounds__(1024 / VPT)
                 const uint32_t code_off = (lane_off[j] / 16u) * (uint32_t)VEC;
                 if constexpr (VEC == 8) {
                     u32x2 w = {codes[0], codes[1]};
-                    __builtin_amdgcn_raw_buffer_store_b64(w, q_out, (int)code_off, 0, kAuxStream);
+                    __builtin_amdgcn_raw_buffer_store_b64(w, q_out, (int)code_off, 0, kAuxStore);
                 } else {
-                    __builtin_amdgcn_raw_buffer_store_b32(codes[0], q_out, (int)code_off, 0, kAuxStream);
+                    __builtin_amdgcn_raw_buffer_store_b32(codes[0], q_out, (int)code_off, 0, kAuxStore);
                 }
             }
         }
-        if constexpr (PF) cur = nxt;
+        if constexpr (PF) {
+            cur = nxt;
+        } else {
+            if (row0 + row_stride < a.tokens) issue_loads(cur, row + row_stride);
+        }
     }
 }
 
