@@ -264,7 +264,7 @@ struct RowLoads {
 // ---------------------------------------------------------------------------------------------
 template <class E, int N, int VPT, int Q, bool WN, bool PF>
 __global__ void __launch_bounds__(1024 / VPT)
-    __attribute__((amdgpu_waves_per_eu(PF ? 4 : (VPT == 1 ? 8 : (VPT == 2 ? 5 : 2))))) row_kernel(const RowArgs a) {
+    __attribute__((amdgpu_waves_per_eu(PF ? 4 : (VPT == 1 ? 8 : (VPT == 2 ? 5 : 3))))) row_kernel(const RowArgs a) {
     constexpr int VEC = E::VEC;
     constexpr int NP = (N == 0) ? 1 : N;
     __shared__ float lds_sum[2][kMaxWavesPerBlock];
@@ -314,18 +314,10 @@ __global__ void __launch_bounds__(1024 / VPT)
     const int64_t row_stride = (int64_t)gridDim.x * a.rows_per_block;
     int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block;
 
-    // The first row's loads go out before anything else touches memory; gamma (shared by every row,
-    // served from L2) is requested behind them and is only needed after the first row reduction.
+    // The first row's loads go out before anything else touches memory.
     RowLoads<NP, VPT> cur;
     issue_loads(cur, row0 + group);
-    __builtin_amdgcn_sched_barrier(0);
-    u32x4 gamma_raw[VPT];
-    {
-        const rsrc_t gr = row_rsrc(a.gamma, 0, row_bytes);
-#pragma unroll
-        for (int j = 0; j < VPT; ++j)
-            gamma_raw[j] = __builtin_amdgcn_raw_buffer_load_b128(gr, (int)lane_off[j], 0, kAuxDefault);
-    }
+    const rsrc_t gamma_rsrc = row_rsrc(a.gamma, 0, row_bytes);
 
     int parity = 0;
     for (; row0 < a.tokens; row0 += row_stride, parity ^= 1) {
@@ -373,6 +365,13 @@ __global__ void __launch_bounds__(1024 / VPT)
                 else sumsq += x[i] * x[i];
             }
         }
+        // gamma (shared by all rows, served from L2) is requested only now: the registers of the row
+        // loads are free again, and the reduction below covers its latency.
+        __builtin_amdgcn_sched_barrier(0);
+        u32x4 gamma_raw[VPT];
+#pragma unroll
+        for (int j = 0; j < VPT; ++j)
+            gamma_raw[j] = __builtin_amdgcn_raw_buffer_load_b128(gamma_rsrc, (int)lane_off[j], 0, kAuxDefault);
         sumsq = row_reduce<OpSum>(sumsq, lds_sum[parity], wave, lane, first_wave, waves_per_row);
         const float rs = 1.0f / __builtin_sqrtf(sumsq / a.hidden_f + a.eps);
 
@@ -383,9 +382,7 @@ __global__ void __launch_bounds__(1024 / VPT)
         for (int j = 0; j < VPT; ++j) {
             float x[VEC], g[VEC], y[VEC];
             E::unpack(xraw[j], x);
-            u32x4 graw = gamma_raw[j];
-            asm volatile("" : "+v"(graw)); // unpack here, per row: hoisting it would put a wait for gamma before the row loads
-            E::unpack(graw, g);
+            E::unpack(gamma_raw[j], g);
 #pragma unroll
             for (int i = 0; i < VEC; ++i) y[i] = x[i] * rs;
             E::unpack(E::pack(y), y);
