@@ -49,7 +49,7 @@ def test_c4_reduced_tokens(cuda_device):
     _case("c4@192", p, r, g, eps, quant)
 
 
-@pytest.mark.parametrize("tokens", [1, 64, 512])
+@pytest.mark.parametrize("tokens", [1, 64, 512, 4096])
 def test_c5_outliers(cuda_device, tokens):
     p, r, g, eps, quant = eager.make_config("c5", tokens=tokens)
     _case("c5@%d" % tokens, p, r, g, eps, quant)
@@ -197,3 +197,60 @@ def test_full_size_c3_properties(cuda_device):
     out2 = tde.reduce_rms(parts, res, gamma, 1e-5, tde.QUANT_FP8_TOKEN, write_norm=True)
     for k in out:
         assert torch.equal(out[k].view(torch.uint8), out2[k].view(torch.uint8)), k         # deterministic run to run
+
+
+def _device_inputs(dev, n, t, h, dtype, sigma, seed, outliers=0):
+    gen = torch.Generator(device=dev).manual_seed(seed)
+    parts = []
+    cols = torch.randperm(h, generator=torch.Generator().manual_seed(seed))[:outliers].to(dev) if outliers else None
+    for _ in range(n):
+        p = torch.randn((t, h), generator=gen, device=dev) * sigma
+        if cols is not None:
+            p[:, cols] *= 100.0
+        parts.append(p.to(dtype))
+    res = torch.randn((t, h), generator=gen, device=dev).to(dtype)
+    gamma = (torch.rand((h,), generator=gen, device=dev) + 0.5).to(dtype)
+    return parts, res, gamma
+
+
+def _device_residual(parts, res):
+    acc = torch.zeros(res.shape, device=res.device)
+    for p in parts:
+        acc = acc + p.float()
+    return (acc.to(res.dtype).float() + res.float()).to(res.dtype)
+
+
+@pytest.mark.parametrize("name,n,t,h,dtype,sigma,eps,quant,outliers", [
+    ("c4", 4, 8192, 7168, torch.bfloat16, 1.0, 1e-6, "fp8_group", 0),
+    ("c5@32768", 4, 32768, 5120, torch.float16, 1.0, 1e-6, "int8_token", 5),
+])
+def test_full_size_c4_c5_properties(cuda_device, name, n, t, h, dtype, sigma, eps, quant, outliers):
+    """BASELINE c4 and the largest c5 at full size.  Inputs are drawn on the device; the residual is checked
+    against the same rank-order sum written with torch device ops, and the quant epilogue against the oracle's
+    quantizer applied on the host to a band of the written normed rows (the whole tensor for the scales)."""
+    import torch_dist_ext_amd as tde
+    print("case", name, flush=True)
+    parts, res, gamma = _device_inputs(cuda_device, n, t, h, dtype, sigma, seed=t, outliers=outliers)
+    mode = {"fp8_group": tde.QUANT_FP8_GROUP, "int8_token": tde.QUANT_INT8_TOKEN}[quant]
+    out = tde.reduce_rms(parts, res, gamma, eps, mode, write_norm=True)
+    torch.cuda.synchronize()
+    assert torch.equal(out["residual_out"].view(torch.int16), _device_residual(parts, res).view(torch.int16))
+    del parts
+    y = out["norm_out"]
+    qmax = 127.0 if quant == "int8_token" else 448.0
+    grp = h if quant == "int8_token" else 128
+    amax = y.float().abs().view(t, h // grp, grp).amax(-1).cpu()
+    assert torch.equal(out["scale"].cpu().view(t, -1), amax / qmax)          # host division: IEEE quotient
+    band = slice(t // 2, t // 2 + 256)
+    yb = y[band].cpu()
+    if quant == "int8_token":
+        q_own, s_own = eager.quant_int8(yb)
+    else:
+        q_own, s_own = eager.quant_fp8(yb, 128)
+    assert bits_equal(q_own, out["q"][band].cpu()) and bits_equal(s_own.reshape(-1), out["scale"][band].cpu().reshape(-1))
+    # every row/group with a non-zero maximum reaches the top code
+    top = out["q"].view(torch.int8 if quant == "int8_token" else torch.float8_e4m3fn).float().abs().view(t, h // grp, grp).amax(-1)
+    assert torch.all((top == qmax) | (out["scale"].view(t, -1) == 0))
+    # rows are normalized: rms(norm/gamma) ~ 1 (second rounding and fp16/bf16 precision allow a small band)
+    rms = torch.sqrt((y.float() / gamma.float()).pow(2).mean(-1))
+    assert torch.all((rms - 1).abs() < 0.02)
