@@ -21,7 +21,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 
 # HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs summarized under
 # profiles/ (scaled by the plain-copy calibration described there); None where not collected.
-TRAFFIC_BYTES = {"c3": 352684544}
+TRAFFIC_BYTES = {"c3": 352694383}
 
 BENCH_CONFIGS = {
     # name: (N, T, H, dtype, sigma, eps, quant)
@@ -171,7 +171,8 @@ def main():
     gbs_job = bytes_per_launch / (wall / args.steps) / 1e9
     achieved = bytes_per_launch / (avg_ms * 1e-3) / 1e9
     out = {
-        "metric": "achieved HBM GB/s, one rank's 8-partial reduce+residual+RMSNorm+per-token fp8 stage",
+        "metric": ("achieved HBM GB/s, one rank's 8-partial reduce+residual+RMSNorm+per-token fp8 stage" if args.config == "c3"
+                   else "achieved HBM GB/s, one rank's %d-partial reduce+residual+RMSNorm stage, quant=%s" % (N, quant)),
         "value": gbs_job, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dt, "data": "synthetic",
