@@ -62,6 +62,7 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     const int64_t lanes = (nvec + vpt - 1) / vpt;
     const int tpr = (int)((lanes + 63) / 64 * 64);
     int rpb = 256 / tpr; // pack short rows so a workgroup has at least four wavefronts
+    if (rpb * tpr > kMaxBlock / vpt) rpb = (kMaxBlock / vpt) / tpr; // never beyond the kernel's launch bound
     if (rpb < 1) rpb = 1;
     if (g_force_rows_per_block > 0 && g_force_rows_per_block * tpr <= kMaxBlock / vpt) rpb = g_force_rows_per_block;
     if (p->tokens > 0 && rpb > p->tokens) rpb = (int)p->tokens;
