@@ -39,7 +39,7 @@ typedef enum tde_status {
     TDE_ESHAPE = 4,     /* hidden*elem not a multiple of 16 bytes, tokens<0, hidden<=0 (impl.h:479-480) */
     TDE_EHIDDEN = 5,    /* hidden larger than the row kernel supports (reference: pkg assert, __init__.py:69) */
     TDE_EALIGN = 6,     /* a buffer is not 16-byte aligned (vec_t alignment, impl.h:208) */
-    TDE_EQUANT = 7,     /* unknown quant mode, or group mode with hidden % 128 != 0 */
+    TDE_EQUANT = 7,     /* unknown quant mode, group mode with hidden % 128 != 0, or a static scale that is not > 0 */
     TDE_EALGO = 8,      /* unknown algorithm, or staged algorithm without a stage buffer */
     TDE_EHIP = 9,       /* HIP runtime error; see tde_last_hip_error() */
     TDE_ERANK = 10,     /* rank outside [0,nranks) */
@@ -57,7 +57,10 @@ typedef enum tde_quant {
     TDE_QUANT_NONE = 0,      /* normed output in the input dtype (the reference's only mode) */
     TDE_QUANT_FP8_TOKEN = 1, /* OCP e4m3 codes, one fp32 scale per row:  scale = rowamax/448 */
     TDE_QUANT_FP8_GROUP = 2, /* OCP e4m3 codes, one fp32 scale per [row, 128-column group]  */
-    TDE_QUANT_INT8_TOKEN = 3 /* int8 codes, one fp32 scale per row:      scale = rowamax/127 */
+    TDE_QUANT_INT8_TOKEN = 3, /* int8 codes, one fp32 scale per row:      scale = rowamax/127 */
+    TDE_QUANT_FP8_STATIC = 4  /* OCP e4m3 codes with a caller-given per-tensor scale (tde_problem.static_scale);
+                                 no scales are written.  The reference carries an unused `scale_factor` field for
+                                 this (impl.h:313). */
 } tde_quant;
 
 typedef enum tde_algo {
@@ -80,7 +83,7 @@ typedef struct tde_problem {
     int64_t tokens;     /* rows; 0 is allowed (no launch) */
     int64_t hidden;     /* columns per row */
     float eps;          /* added to mean(x^2) before the reciprocal square root */
-    int32_t reserved;
+    float static_scale; /* TDE_QUANT_FP8_STATIC: code = e4m3(clamp(y / static_scale, +-448)); must be > 0 and finite */
 } tde_problem;
 
 typedef struct tde_buffers {
@@ -96,7 +99,7 @@ typedef struct tde_buffers {
     void *norm_out;    /* may be null when quant != NONE and write_norm == 0 */
     const void *gamma; /* [hidden] of `dtype` */
     void *q_out;       /* [tokens, hidden] bytes (fp8 e4m3 / int8); null when quant == NONE */
-    float *scale_out;  /* [tokens] or [tokens, hidden/128] fp32; null when quant == NONE */
+    float *scale_out;  /* [tokens] or [tokens, hidden/128] fp32; null when quant == NONE or FP8_STATIC */
     void *stage;       /* [tokens, hidden] of `dtype`; required for TDE_ALGO_STAGED */
 } tde_buffers;
 

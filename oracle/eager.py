@@ -16,7 +16,7 @@ all_reduce_fusion_impl.h:26,313 are unused) and its tests assert nothing, so:
            order-sensitivity vector, an integer-arithmetic RNE restatement (oracle/tde_oracle.c),
            the reference's fp64 CPU check (test/unit_test.cpp:175-217, restated) and, where it
            builds, oracle/_ref (that function compiled from the reference's own file).
-  PARITY UNPINNED by the reference: quant_fp8 / quant_int8.  Their definition is this build's own
+  PARITY UNPINNED by the reference: quant_fp8 / quant_int8 / quant_fp8_static.  Their definition is this build's own
            (scale = amax/448 resp. amax/127, RNE codes, clamp); they are pinned only against the
            mathematics: a textbook e4m3 encoder over all codes and midpoints, max-code and
            half-step dequantization properties, ties-to-even for int8.
@@ -73,14 +73,20 @@ def quant_fp8(y: torch.Tensor, group=None):
     return scaled.to(torch.float8_e4m3fn), scale
 
 
+def quant_fp8_static(y: torch.Tensor, scale: float):
+    """OCP e4m3 codes with a caller-given per-tensor scale (fp32): e4m3(clamp(float(y)/scale, +-448))."""
+    s = torch.tensor(scale, dtype=torch.float32)
+    return (y.float() / s).clamp(-FP8_E4M3_MAX, FP8_E4M3_MAX).to(torch.float8_e4m3fn)
+
+
 def quant_int8(y: torch.Tensor):
     """Dynamic symmetric int8 per row: scale = amax/127, code = clamp(round_half_even(y/scale), +-127)."""
     scale, scaled = _scales_and_scaled(y, INT8_MAX, None)
     return torch.round(scaled).to(torch.int8), scale.view(-1)
 
 
-def reduce_rms(parts, residual_in, gamma, eps, quant="none"):
-    """The whole stage.  quant in {"none", "fp8_token", "fp8_group", "int8_token"}.
+def reduce_rms(parts, residual_in, gamma, eps, quant="none", static_scale=None):
+    """The whole stage.  quant in {"none", "fp8_token", "fp8_group", "int8_token", "fp8_static"}.
     Returns dict(residual_out, norm_out[, q, scale])."""
     residual_out = reduce_residual(parts, residual_in)
     norm_out = rmsnorm(residual_out, gamma, eps)
@@ -91,6 +97,8 @@ def reduce_rms(parts, residual_in, gamma, eps, quant="none"):
         out["q"], out["scale"] = quant_fp8(norm_out, GROUP)
     elif quant == "int8_token":
         out["q"], out["scale"] = quant_int8(norm_out)
+    elif quant == "fp8_static":
+        out["q"] = quant_fp8_static(norm_out, static_scale)
     elif quant != "none":
         raise ValueError(quant)
     return out

@@ -5,7 +5,7 @@ from torch_dist_ext_amd import _capi
 
 DTYPE_CODE = {torch.bfloat16: _capi.BF16, torch.float16: _capi.F16, torch.float32: _capi.F32}
 QUANT_CODE = {"none": _capi.QUANT_NONE, "fp8_token": _capi.QUANT_FP8_TOKEN, "fp8_group": _capi.QUANT_FP8_GROUP,
-              "int8_token": _capi.QUANT_INT8_TOKEN}
+              "int8_token": _capi.QUANT_INT8_TOKEN, "fp8_static": _capi.QUANT_FP8_STATIC}
 
 
 def ordered_bits(t: torch.Tensor) -> torch.Tensor:
@@ -34,7 +34,7 @@ def bits_equal(a: torch.Tensor, b: torch.Tensor) -> bool:
 
 
 def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, write_norm=None, use_table=False,
-            rank=0, device="cuda:0"):
+            rank=0, device="cuda:0", static_scale=0.0):
     """Run the HIP path through the C ABI (tde_reduce_rms) on CPU inputs; returns CPU outputs.
     parts: [N,T,H] tensor or list of N [T,H] tensors."""
     dev = torch.device(device)
@@ -54,10 +54,11 @@ def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, wri
     if qm:
         d_q = torch.empty((T, H), dtype=torch.uint8, device=dev)
         nscale = T * (H // 128) if quant == "fp8_group" else T
-        d_scale = torch.empty((nscale,), dtype=torch.float32, device=dev)
+        if quant != "fp8_static":
+            d_scale = torch.empty((nscale,), dtype=torch.float32, device=dev)
     d_stage = torch.empty_like(d_res) if algo == _capi.ALGO_STAGED else None
     prob = _capi.make_problem(DTYPE_CODE[dtype], n, T, H, eps, quant=qm, algo=algo, write_norm=int(bool(write_norm)),
-                              rank=rank)
+                              rank=rank, static_scale=static_scale)
     ptrs = [p.data_ptr() for p in d_parts]
     table = None
     d_table = None
@@ -79,8 +80,9 @@ def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, wri
     if qm:
         q = d_q.cpu()
         out["q"] = q.view(torch.int8) if quant == "int8_token" else q.view(torch.float8_e4m3fn)
-        sc = d_scale.cpu()
-        out["scale"] = sc.view(T, H // 128) if quant == "fp8_group" else sc
+        if d_scale is not None:
+            sc = d_scale.cpu()
+            out["scale"] = sc.view(T, H // 128) if quant == "fp8_group" else sc
     return out
 
 

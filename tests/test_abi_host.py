@@ -49,6 +49,7 @@ def _plan(**kw):
     (dict(hidden=8200), _capi.EHIDDEN),     # beyond 1024 vectors per row (the reference asserts hidden <= 8192)
     (dict(dtype=_capi.F32, hidden=4100), _capi.EHIDDEN),
     (dict(quant=9), _capi.EQUANT), (dict(quant=_capi.QUANT_FP8_GROUP, hidden=1032), _capi.EQUANT),
+    (dict(quant=_capi.QUANT_FP8_STATIC), _capi.EQUANT), (dict(quant=_capi.QUANT_FP8_STATIC, static_scale=-2.0), _capi.EQUANT),
     (dict(algo=5), _capi.EALGO), (dict(rank=8), _capi.ERANK), (dict(rank=-1), _capi.ERANK),
 ])
 def test_plan_rejects(kw, status):

@@ -7,7 +7,7 @@ import torch
 from oracle import eager
 from torch_dist_ext_amd import _capi
 
-from helpers import bits_equal, check_against_oracle, run_hip
+from helpers import bits_equal, check_against_oracle, run_hip, ulp_distance
 
 pytestmark = pytest.mark.gpu
 
@@ -254,3 +254,78 @@ def test_full_size_c4_c5_properties(cuda_device, name, n, t, h, dtype, sigma, ep
     # rows are normalized: rms(norm/gamma) ~ 1 (second rounding and fp16/bf16 precision allow a small band)
     rms = torch.sqrt((y.float() / gamma.float()).pow(2).mean(-1))
     assert torch.all((rms - 1).abs() < 0.02)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("scale", [0.0078125, 0.013, 1.7])
+def test_static_scale_fp8(cuda_device, dtype, scale):
+    """Caller-given per-tensor scale: codes must be the oracle's static quantizer applied to the kernel's own
+    normed rows, bit for bit (values beyond 448*scale saturate to the top code)."""
+    p, r, g = eager.make_inputs(4, 45, 2048, dtype, 1.0, seed=41)
+    print("case static", dtype, scale, flush=True)
+    want = eager.reduce_rms(p, r, g, 1e-6, "fp8_static", static_scale=scale)
+    got = run_hip(p, r, g, 1e-6, "fp8_static", static_scale=scale)
+    assert "scale" not in got
+    check_against_oracle({k: got[k] for k in ("residual_out", "norm_out")}, want, "none", gamma=g, eps=1e-6)
+    assert bits_equal(got["q"], eager.quant_fp8_static(got["norm_out"], scale))
+    assert int(ulp_distance(got["q"], want["q"]).max()) <= 1
+    got2 = run_hip(p, r, g, 1e-6, "fp8_static", static_scale=scale, write_norm=False)
+    assert bits_equal(got2["q"], got["q"])
+
+
+def test_static_scale_is_validated(cuda_device):
+    p, r, g = eager.make_inputs(2, 4, 256, torch.bfloat16, 1.0, seed=42)
+    for bad in (0.0, -1.0, float("inf"), float("nan")):
+        with pytest.raises(_capi.TdeError) as e:
+            run_hip(p, r, g, 1e-6, "fp8_static", static_scale=bad)
+        assert e.value.status == _capi.EQUANT
+
+
+def test_hip_graph_replays_match_eager(cuda_device):
+    """The launch allocates nothing and synchronizes nothing, so it can be captured.  Replays are checked
+    against eager launches, with new input contents and eager work between the replays."""
+    dev = cuda_device
+    n, t, h = 8, 128, 4096
+    parts = [torch.empty((t, h), dtype=torch.bfloat16, device=dev) for _ in range(n)]
+    res = torch.empty((t, h), dtype=torch.bfloat16, device=dev)
+    gamma = torch.empty((h,), dtype=torch.bfloat16, device=dev)
+    outs = {k: torch.empty((t, h), dtype=torch.bfloat16, device=dev) for k in ("res_out", "norm")}
+    q = torch.empty((t, h), dtype=torch.uint8, device=dev)
+    sc = torch.empty((t,), dtype=torch.float32, device=dev)
+    prob = _capi.make_problem(_capi.BF16, n, t, h, 1e-5, quant=_capi.QUANT_FP8_TOKEN, write_norm=1)
+
+    def launch(stream):
+        _capi.reduce_rms(prob, [p.data_ptr() for p in parts], res.data_ptr(), outs["res_out"].data_ptr(), gamma.data_ptr(),
+                         norm_out=outs["norm"].data_ptr(), q_out=q.data_ptr(), scale_out=sc.data_ptr(), stream=stream)
+
+    def fill(seed):
+        cp, cr, cg = eager.make_inputs(n, t, h, torch.bfloat16, 0.5, seed=seed)
+        for i in range(n):
+            parts[i].copy_(cp[i])
+        res.copy_(cr)
+        gamma.copy_(cg)
+        return cp, cr, cg
+
+    fill(1)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch(side.cuda_stream)            # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        launch(torch.cuda.current_stream().cuda_stream)
+    for seed in (2, 3, 4):
+        cp, cr, cg = fill(seed)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = {"residual_out": outs["res_out"].cpu(), "norm_out": outs["norm"].cpu(),
+               "q": q.cpu().view(torch.float8_e4m3fn), "scale": sc.cpu()}
+        for v in (outs["res_out"], outs["norm"], q, sc):
+            v.zero_()                        # eager work between replays
+        launch(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        assert bits_equal(outs["res_out"].cpu(), got["residual_out"]) and bits_equal(outs["norm"].cpu(), got["norm_out"])
+        assert bits_equal(q.cpu(), got["q"].view(torch.uint8)) and bits_equal(sc.cpu(), got["scale"])
+        check_against_oracle(got, eager.reduce_rms(cp, cr, cg, 1e-5, "fp8_token"), "fp8_token", gamma=cg, eps=1e-5)

@@ -93,3 +93,46 @@ def test_error_paths_raise(tde, cuda_device):
     y = torch.zeros((4, 8200), dtype=torch.bfloat16, device=cuda_device)
     with pytest.raises(AssertionError):
         tde.allreduce_rms(0, 2, y, y, torch.ones(8200, dtype=torch.bfloat16, device=cuda_device), 1e-6, ws)
+
+
+def test_workspace_table_is_uploaded_once_and_ops_trace(tde, cuda_device):
+    """get_workspace hands out one cached device table (no per-call host-to-device copy), and the custom
+    ops run under torch.compile (aot_eager: traced through their fake implementations, no code generation)."""
+    world_size, tokens, hidden, eps, rank = 2, 16, 1024, 1e-6, 0
+    p, r, g = eager.make_inputs(world_size, tokens, hidden, torch.bfloat16, 1.0, seed=51)
+    tde.setup_env(rank, world_size, max_size_in_bytes=tokens * hidden * 2)
+    tde.set_peer_partial(1, p[1].to(cuda_device))
+    x = p[0].to(cuda_device)
+    ws1 = tde.get_workspace(x)
+    ws2 = tde.get_workspace(x)
+    assert ws1.data_ptr() == ws2.data_ptr()
+    rd, gd = r.to(cuda_device), g.to(cuda_device)
+
+    def step(x, rd, gd, ws):
+        n, ro = torch.ops.torch_dist_ext.allreduce_rms(rank, world_size, x, rd, gd, eps, ws)
+        return n * 2, ro
+
+    want = eager.reduce_rms(p, r, g, eps)
+    compiled = torch.compile(step, backend="aot_eager", fullgraph=True)
+    n2, ro = compiled(x, rd, gd, ws1)
+    torch.cuda.synchronize()
+    assert bits_equal(ro.cpu(), want["residual_out"])
+    assert bits_equal(n2.cpu(), (want["norm_out"] * 2))
+
+
+def test_static_quant_op(tde, cuda_device):
+    p, r, g = eager.make_inputs(4, 20, 1024, torch.bfloat16, 1.0, seed=52)
+    parts = [p[i].to(cuda_device) for i in range(4)]
+    out = tde.reduce_rms(parts, r.to(cuda_device), g.to(cuda_device), 1e-6, tde.QUANT_FP8_STATIC, write_norm=True,
+                         static_scale=0.01)
+    torch.cuda.synchronize()
+    assert "scale" not in out
+    assert bits_equal(out["q"].cpu(), eager.quant_fp8_static(out["norm_out"].cpu(), 0.01))
+    tde.setup_env(0, 4, max_size_in_bytes=20 * 1024 * 2)
+    for k in range(1, 4):
+        tde.set_peer_partial(k, parts[k])
+    ws = tde.get_workspace(parts[0])
+    q, s, ro, no = torch.ops.torch_dist_ext.allreduce_rms_quant(0, 4, parts[0], r.to(cuda_device), g.to(cuda_device), 1e-6, ws,
+                                                               tde.QUANT_FP8_STATIC, False, 0.01)
+    torch.cuda.synchronize()
+    assert s.numel() == 0 and no.numel() == 0 and bits_equal(q.cpu(), out["q"].cpu())

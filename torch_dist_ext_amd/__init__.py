@@ -18,8 +18,8 @@ from typing import Tuple
 import torch
 
 from . import _capi
-from ._capi import (ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, QUANT_FP8_GROUP, QUANT_FP8_TOKEN, QUANT_INT8_TOKEN, QUANT_NONE,
-                    QUANT_GROUP)
+from ._capi import (ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, QUANT_FP8_GROUP, QUANT_FP8_STATIC, QUANT_FP8_TOKEN, QUANT_INT8_TOKEN,
+                    QUANT_NONE, QUANT_GROUP)
 
 this_dir = os.path.dirname(os.path.abspath(__file__))
 filename = os.path.join(this_dir, "libtorch_dist_ext.so")
@@ -35,7 +35,8 @@ allreduce_rms_fusion_impl = torch.ops.torch_dist_ext.allreduce_rms_fusion
 allreduce_rms_quant_fusion_impl = torch.ops.torch_dist_ext.allreduce_rms_quant_fusion
 reduce_rms_local_impl = torch.ops.torch_dist_ext.reduce_rms_local
 
-QUANT_MODES = {"none": QUANT_NONE, "fp8_token": QUANT_FP8_TOKEN, "fp8_group": QUANT_FP8_GROUP, "int8_token": QUANT_INT8_TOKEN}
+QUANT_MODES = {"none": QUANT_NONE, "fp8_token": QUANT_FP8_TOKEN, "fp8_group": QUANT_FP8_GROUP, "int8_token": QUANT_INT8_TOKEN,
+               "fp8_static": QUANT_FP8_STATIC}
 
 
 class CommProcess:
@@ -122,6 +123,8 @@ def _quant_out_shapes(allreduce_in: torch.Tensor, quant_mode: int):
     lead = tuple(allreduce_in.shape[:-1])
     if quant_mode == QUANT_FP8_GROUP:
         scale_shape = lead + (hidden // QUANT_GROUP,)
+    elif quant_mode == QUANT_FP8_STATIC:
+        scale_shape = (0,)   # the scale is the caller's; nothing is written
     else:
         scale_shape = lead
     q_dtype = torch.int8 if quant_mode == QUANT_INT8_TOKEN else torch.float8_e4m3fn
@@ -131,19 +134,20 @@ def _quant_out_shapes(allreduce_in: torch.Tensor, quant_mode: int):
 @torch.library.custom_op("torch_dist_ext::allreduce_rms_quant", mutates_args=[])
 def allreduce_rms_quant(rank: int, nranks: int, allreduce_in: torch.Tensor, residual_in: torch.Tensor,
                         rms_gamma: torch.Tensor, eps: float, workspace: torch.Tensor, quant_mode: int,
-                        write_norm: bool) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+                        write_norm: bool, static_scale: float = 0.0) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """Quantizing form of allreduce_rms: returns (codes, scales, residual_out, norm_out).
-    quant_mode is one of QUANT_FP8_TOKEN / QUANT_FP8_GROUP / QUANT_INT8_TOKEN; norm_out has zero
-    elements unless write_norm."""
+    quant_mode is one of QUANT_FP8_TOKEN / QUANT_FP8_GROUP / QUANT_INT8_TOKEN / QUANT_FP8_STATIC; norm_out has
+    zero elements unless write_norm; scales has zero elements for QUANT_FP8_STATIC (static_scale is the scale)."""
     assert allreduce_in.shape[-1] <= 8192
-    assert quant_mode in (QUANT_FP8_TOKEN, QUANT_FP8_GROUP, QUANT_INT8_TOKEN)
+    assert quant_mode in (QUANT_FP8_TOKEN, QUANT_FP8_GROUP, QUANT_INT8_TOKEN, QUANT_FP8_STATIC)
     q_dtype, scale_shape = _quant_out_shapes(allreduce_in, quant_mode)
     q_out = torch.empty(allreduce_in.shape, dtype=q_dtype, device=allreduce_in.device)
     scale_out = torch.empty(scale_shape, dtype=torch.float32, device=allreduce_in.device)
     residual_out = torch.empty_like(residual_in)
     norm_out = torch.empty_like(allreduce_in) if write_norm else None
     allreduce_rms_quant_fusion_impl(rank, nranks, allreduce_in, residual_in, rms_gamma, residual_out, norm_out, q_out,
-                                    scale_out, eps, workspace, quant_mode)
+                                    scale_out if quant_mode != QUANT_FP8_STATIC else None, eps, workspace, quant_mode,
+                                    static_scale)
     if norm_out is None:
         norm_out = allreduce_in.new_empty((0,))
     return q_out, scale_out, residual_out, norm_out
@@ -152,7 +156,7 @@ def allreduce_rms_quant(rank: int, nranks: int, allreduce_in: torch.Tensor, resi
 @torch.library.register_fake("torch_dist_ext::allreduce_rms_quant")
 def allreduce_rms_quant_fake(rank: int, nranks: int, allreduce_in: torch.Tensor, residual_in: torch.Tensor,
                              rms_gamma: torch.Tensor, eps: float, workspace: torch.Tensor, quant_mode: int,
-                             write_norm: bool) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+                             write_norm: bool, static_scale: float = 0.0) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     q_dtype, scale_shape = _quant_out_shapes(allreduce_in, quant_mode)
     q_out = torch.empty(allreduce_in.shape, dtype=q_dtype, device=allreduce_in.device)
     scale_out = torch.empty(scale_shape, dtype=torch.float32, device=allreduce_in.device)
@@ -161,7 +165,8 @@ def allreduce_rms_quant_fake(rank: int, nranks: int, allreduce_in: torch.Tensor,
     return q_out, scale_out, residual_out, norm_out
 
 
-def reduce_rms(partials, residual_in, rms_gamma, eps, quant_mode=QUANT_NONE, write_norm=None, algo=ALGO_AUTO, stage=None):
+def reduce_rms(partials, residual_in, rms_gamma, eps, quant_mode=QUANT_NONE, write_norm=None, algo=ALGO_AUTO, stage=None,
+               static_scale=0.0):
     """One rank's stage with the N partials passed as a list of N [tokens, hidden] GPU tensors.
 
     Returns a dict with residual_out and, depending on the mode, norm_out / q / scale."""
@@ -174,12 +179,14 @@ def reduce_rms(partials, residual_in, rms_gamma, eps, quant_mode=QUANT_NONE, wri
     if quant_mode != QUANT_NONE:
         q_dtype, scale_shape = _quant_out_shapes(ref, quant_mode)
         q_out = torch.empty(ref.shape, dtype=q_dtype, device=ref.device)
-        scale_out = torch.empty(scale_shape, dtype=torch.float32, device=ref.device)
-        out["q"], out["scale"] = q_out, scale_out
+        out["q"] = q_out
+        if quant_mode != QUANT_FP8_STATIC:
+            scale_out = torch.empty(scale_shape, dtype=torch.float32, device=ref.device)
+            out["scale"] = scale_out
     if algo == ALGO_STAGED and stage is None:
         stage = torch.empty_like(ref)
     reduce_rms_local_impl(list(partials), residual_in, rms_gamma, out["residual_out"], norm_out, q_out, scale_out, eps,
-                          quant_mode, algo, stage)
+                          quant_mode, algo, stage, static_scale)
     if norm_out is not None:
         out["norm_out"] = norm_out
     return out

@@ -12,7 +12,7 @@ QUANT_GROUP = 128
 
 OK, EINVAL, ENRANKS, EDTYPE, ESHAPE, EHIDDEN, EALIGN, EQUANT, EALGO, EHIP, ERANK, ENOMEM = range(12)
 BF16, F16, F32 = 0, 1, 2
-QUANT_NONE, QUANT_FP8_TOKEN, QUANT_FP8_GROUP, QUANT_INT8_TOKEN = 0, 1, 2, 3
+QUANT_NONE, QUANT_FP8_TOKEN, QUANT_FP8_GROUP, QUANT_INT8_TOKEN, QUANT_FP8_STATIC = 0, 1, 2, 3, 4
 ALGO_AUTO, ALGO_FUSED, ALGO_STAGED = 0, 1, 2
 
 # Every symbol include/tde_abi.h declares.
@@ -27,7 +27,7 @@ class Problem(ctypes.Structure):
     _fields_ = [
         ("dtype", ctypes.c_int32), ("nranks", ctypes.c_int32), ("rank", ctypes.c_int32), ("quant", ctypes.c_int32),
         ("algo", ctypes.c_int32), ("write_norm", ctypes.c_int32), ("tokens", ctypes.c_int64), ("hidden", ctypes.c_int64),
-        ("eps", ctypes.c_float), ("reserved", ctypes.c_int32),
+        ("eps", ctypes.c_float), ("static_scale", ctypes.c_float),
     ]
 
 
@@ -107,9 +107,10 @@ def check(status):
         raise TdeError(status, text)
 
 
-def make_problem(dtype, nranks, tokens, hidden, eps, quant=QUANT_NONE, algo=ALGO_AUTO, write_norm=0, rank=0):
+def make_problem(dtype, nranks, tokens, hidden, eps, quant=QUANT_NONE, algo=ALGO_AUTO, write_norm=0, rank=0,
+                 static_scale=0.0):
     return Problem(dtype=dtype, nranks=nranks, rank=rank, quant=quant, algo=algo, write_norm=int(write_norm),
-                   tokens=tokens, hidden=hidden, eps=eps, reserved=0)
+                   tokens=tokens, hidden=hidden, eps=eps, static_scale=static_scale)
 
 
 def plan(problem):

@@ -47,7 +47,8 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     if (p->rank < 0 || p->rank >= p->nranks) return TDE_ERANK;
     if (p->tokens < 0 || p->hidden <= 0) return TDE_ESHAPE;
     if ((p->hidden * eb) % 16 != 0) return TDE_ESHAPE;
-    if (p->quant < TDE_QUANT_NONE || p->quant > TDE_QUANT_INT8_TOKEN) return TDE_EQUANT;
+    if (p->quant < TDE_QUANT_NONE || p->quant > TDE_QUANT_FP8_STATIC) return TDE_EQUANT;
+    if (p->quant == TDE_QUANT_FP8_STATIC && !(p->static_scale > 0.0f && p->static_scale <= 3.0e38f)) return TDE_EQUANT;
     if (p->quant == TDE_QUANT_FP8_GROUP && p->hidden % TDE_QUANT_GROUP != 0) return TDE_EQUANT;
     if (p->algo < TDE_ALGO_AUTO || p->algo > TDE_ALGO_STAGED) return TDE_EALGO;
     const int vec = 16 / eb;
@@ -96,6 +97,7 @@ int64_t algorithmic_bytes(const tde_problem *p, int64_t *scale_elems) {
     case TDE_QUANT_FP8_TOKEN:
     case TDE_QUANT_INT8_TOKEN: scales = T; out = T * H + 4 * scales; break;
     case TDE_QUANT_FP8_GROUP: scales = T * (H / TDE_QUANT_GROUP); out = T * H + 4 * scales; break;
+    case TDE_QUANT_FP8_STATIC: out = T * H; break;
     }
     if (p->quant != TDE_QUANT_NONE && p->write_norm) out += T * H * e;
     if (scale_elems) *scale_elems = scales;
@@ -136,7 +138,7 @@ const char *tde_status_string(int status) {
     case TDE_ESHAPE: return "bad shape: hidden*elem_size must be a positive multiple of 16 bytes, tokens >= 0";
     case TDE_EHIDDEN: return "hidden too large for the one-pass row kernel (max 1024 16-byte vectors per row: 8192 bf16/f16, 4096 f32)";
     case TDE_EALIGN: return "buffer not 16-byte aligned";
-    case TDE_EQUANT: return "bad quant mode, or per-group quant with hidden not a multiple of 128";
+    case TDE_EQUANT: return "bad quant mode, per-group quant with hidden not a multiple of 128, or static scale not > 0";
     case TDE_EALGO: return "bad algorithm, or staged algorithm without a stage buffer";
     case TDE_EHIP: return "HIP runtime error (see tde_last_hip_error)";
     case TDE_ERANK: return "rank outside [0, nranks)";
@@ -200,7 +202,8 @@ int tde_reduce_rms(const tde_problem *p, const tde_buffers *b, void *hip_stream)
     }
     if (!b->residual_in || !b->residual_out || !b->gamma) return TDE_EINVAL;
     if (wn && !b->norm_out) return TDE_EINVAL;
-    if (quant && (!b->q_out || !b->scale_out)) return TDE_EINVAL;
+    if (quant && !b->q_out) return TDE_EINVAL;
+    if (quant && p->quant != TDE_QUANT_FP8_STATIC && !b->scale_out) return TDE_EINVAL;
     if (staged && !b->stage) return TDE_EALGO;
     if (!aligned16(b->residual_in) || !aligned16(b->residual_out) || !aligned16(b->gamma) ||
         !aligned16(b->norm_out) || !aligned16(b->stage) || !aligned16(b->partial_table))
@@ -226,6 +229,7 @@ int tde_reduce_rms(const tde_problem *p, const tde_buffers *b, void *hip_stream)
     a.rows_per_block = g.rows_per_block;
     a.eps = p->eps;
     a.hidden_f = (float)p->hidden;
+    a.static_scale = p->static_scale;
 
     int n = p->nranks;
     hipError_t e = hipSuccess;

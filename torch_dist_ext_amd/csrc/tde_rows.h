@@ -12,6 +12,7 @@
 //   per-token fp8 : scale = amax|y| / 448, code = e4m3( clamp(float(y)/scale, +-448) )
 //   per-group fp8 : the same over each 128-column group
 //   per-token int8: scale = amax|y| / 127, code = clamp(rne(float(y)/scale), +-127)
+//   static fp8    : code = e4m3( clamp(float(y)/static_scale, +-448) ), no scale written
 //
 // Included by one translation unit per element type; nothing here is exported.
 #pragma once
@@ -51,6 +52,7 @@ struct RowArgs {
     int32_t rows_per_block;
     float eps;
     float hidden_f;
+    float static_scale;
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -393,7 +395,7 @@ __global__ void __launch_bounds__(1024 / VPT)
                 const rsrc_t norm_out = row_rsrc(a.norm_out, row_byte, bytes);
                 rsrc_store16(norm_out, lane_off[j], yraw[j]);
             }
-            if constexpr (Q != TDE_QUANT_NONE) {
+            if constexpr (Q != TDE_QUANT_NONE && Q != TDE_QUANT_FP8_STATIC) {
                 E::unpack(yraw[j], y);
                 float m = 0.0f;
 #pragma unroll
@@ -419,6 +421,9 @@ __global__ void __launch_bounds__(1024 / VPT)
                         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, scale[j]), sc_out,
                                                               (int)((lane_off[j] / 16u / LANES_PER_GROUP) * 4u), 0, kAuxDefault);
                 }
+            } else if constexpr (Q == TDE_QUANT_FP8_STATIC) {
+#pragma unroll
+                for (int j = 0; j < VPT; ++j) scale[j] = a.static_scale;
             } else {
                 float m = amax[0];
 #pragma unroll
@@ -535,6 +540,8 @@ hipError_t launch_rows_nvp(int q, bool wn, const RowArgs &a, const Geometry &g, 
         if (wn) { TDE_LAUNCH(TDE_QUANT_FP8_GROUP, true) } else { TDE_LAUNCH(TDE_QUANT_FP8_GROUP, false) }
     case TDE_QUANT_INT8_TOKEN:
         if (wn) { TDE_LAUNCH(TDE_QUANT_INT8_TOKEN, true) } else { TDE_LAUNCH(TDE_QUANT_INT8_TOKEN, false) }
+    case TDE_QUANT_FP8_STATIC:
+        if (wn) { TDE_LAUNCH(TDE_QUANT_FP8_STATIC, true) } else { TDE_LAUNCH(TDE_QUANT_FP8_STATIC, false) }
     }
 #undef TDE_LAUNCH
     return hipErrorInvalidValue;

@@ -95,12 +95,18 @@ public:
     }
 
     // uint8 device tensor of (3*world_size+5) pointers, layout of src/ops/all_reduce_fusion.cpp:159-169.
+    // The table never changes after construction, so it is uploaded once and the same device
+    // tensor is handed out afterwards (the reference rebuilds and copies it on every call,
+    // src/ops/all_reduce_fusion.cpp:159-173): no host-to-device copy in steady state, which also
+    // keeps the call legal while a HIP graph is being captured.
     Tensor get_workspace(const Tensor &ref) {
+        if (table_.defined() && table_.device() == ref.device()) return table_;
         const int64_t entries = 3 * world_size_ + 5;
         auto host = at::empty({entries * (int64_t)sizeof(void *)}, at::TensorOptions().dtype(at::kByte).device(at::kCPU));
         check_status(tde_workspace_fill_table(ws_, reinterpret_cast<void **>(host.data_ptr()), (int32_t)entries),
                      "get_workspace");
-        return host.to(ref.device());
+        table_ = host.to(ref.device());
+        return table_;
     }
 
     // ---- emulation-only additions (no counterpart in the reference) -----------------------------
@@ -135,6 +141,7 @@ private:
     int device_ = 0;
     bool opened_ = false;
     tde_workspace *ws_ = nullptr;
+    Tensor table_;
 };
 
 namespace {
@@ -165,15 +172,22 @@ void fill_common(Call &c, int64_t rank, int64_t nranks, const Tensor &allreduce_
 }
 
 void fill_quant(Call &c, int64_t quant_mode, const Tensor &like, const c10::optional<Tensor> &norm_out,
-                const c10::optional<Tensor> &q_out, const c10::optional<Tensor> &scale_out) {
+                const c10::optional<Tensor> &q_out, const c10::optional<Tensor> &scale_out, double static_scale = 0.0) {
     c.p.quant = (int32_t)quant_mode;
+    c.p.static_scale = (float)static_scale;
     if (norm_out.has_value() && norm_out->defined()) {
         check_row_tensor(*norm_out, like, "norm_out");
         c.b.norm_out = norm_out->data_ptr();
         c.p.write_norm = 1;
     }
-    if (quant_mode != TDE_QUANT_NONE) {
-        TORCH_CHECK(q_out.has_value() && scale_out.has_value(), "quant modes need q_out and scale_out");
+    if (quant_mode == TDE_QUANT_FP8_STATIC) {
+        TORCH_CHECK(q_out.has_value() && q_out->defined(), "static fp8 quant needs q_out");
+        TORCH_CHECK(q_out->is_cuda() && q_out->is_contiguous() && q_out->element_size() == 1 && q_out->numel() == like.numel(),
+                    "q_out must be a contiguous 1-byte GPU tensor with allreduce_in's numel");
+        c.b.q_out = q_out->data_ptr();
+    } else if (quant_mode != TDE_QUANT_NONE) {
+        TORCH_CHECK(q_out.has_value() && scale_out.has_value() && q_out->defined() && scale_out->defined(),
+                    "dynamic quant modes need q_out and scale_out");
         TORCH_CHECK(q_out->is_cuda() && q_out->is_contiguous() && q_out->element_size() == 1 && q_out->numel() == like.numel(),
                     "q_out must be a contiguous 1-byte GPU tensor with allreduce_in's numel");
         const int64_t tokens = c.p.tokens;
@@ -214,11 +228,12 @@ void allreduce_rms_fusion(int64_t rank, int64_t nranks, Tensor &allreduce_in, Te
 
 // Quantizing variant behind the same workspace protocol.
 void allreduce_rms_quant_fusion(int64_t rank, int64_t nranks, Tensor &allreduce_in, Tensor &residual_in, Tensor &rms_gamma,
-                                Tensor &residual_out, c10::optional<Tensor> norm_out, Tensor &q_out, Tensor &scale_out,
-                                double eps, Tensor &workspace, int64_t quant_mode) {
+                                Tensor &residual_out, c10::optional<Tensor> norm_out, Tensor &q_out,
+                                c10::optional<Tensor> scale_out, double eps, Tensor &workspace, int64_t quant_mode,
+                                double static_scale) {
     Call c;
     fill_common(c, rank, nranks, allreduce_in, residual_in, rms_gamma, residual_out, eps);
-    fill_quant(c, quant_mode, allreduce_in, norm_out, q_out, scale_out);
+    fill_quant(c, quant_mode, allreduce_in, norm_out, q_out, scale_out, static_scale);
     TORCH_CHECK(workspace.is_cuda() && workspace.scalar_type() == at::kByte && workspace.is_contiguous() &&
                     workspace.numel() >= (3 * nranks + 5) * (int64_t)sizeof(void *),
                 "workspace must be the uint8 GPU pointer table returned by get_workspace for this world size");
@@ -231,11 +246,11 @@ void allreduce_rms_quant_fusion(int64_t rank, int64_t nranks, Tensor &allreduce_
 // The same stage with the N partials given directly as N tensors (no workspace object).
 void reduce_rms_local(std::vector<Tensor> partials, Tensor &residual_in, Tensor &rms_gamma, Tensor &residual_out,
                       c10::optional<Tensor> norm_out, c10::optional<Tensor> q_out, c10::optional<Tensor> scale_out,
-                      double eps, int64_t quant_mode, int64_t algo, c10::optional<Tensor> stage) {
+                      double eps, int64_t quant_mode, int64_t algo, c10::optional<Tensor> stage, double static_scale) {
     TORCH_CHECK(!partials.empty() && partials.size() <= TDE_MAX_RANKS, "reduce_rms_local: 2, 4 or 8 partials expected");
     Call c;
     fill_common(c, 0, (int64_t)partials.size(), partials[0], residual_in, rms_gamma, residual_out, eps);
-    fill_quant(c, quant_mode, partials[0], norm_out, q_out, scale_out);
+    fill_quant(c, quant_mode, partials[0], norm_out, q_out, scale_out, static_scale);
     for (size_t r = 0; r < partials.size(); ++r) {
         check_row_tensor(partials[r], partials[0], "partial");
         c.b.partial[r] = partials[r].data_ptr();
@@ -265,10 +280,11 @@ TORCH_LIBRARY(torch_dist_ext, m) {
     m.def("allreduce_rms_fusion(SymInt rank, SymInt nranks, Tensor allreduce_in, Tensor residual_in, Tensor rms_gamma, "
           "Tensor residual_out, Tensor norm_out, float eps, Tensor workspace) -> ()");
     m.def("allreduce_rms_quant_fusion(SymInt rank, SymInt nranks, Tensor allreduce_in, Tensor residual_in, Tensor rms_gamma, "
-          "Tensor residual_out, Tensor? norm_out, Tensor q_out, Tensor scale_out, float eps, Tensor workspace, "
-          "int quant_mode) -> ()");
+          "Tensor residual_out, Tensor? norm_out, Tensor q_out, Tensor? scale_out, float eps, Tensor workspace, "
+          "int quant_mode, float static_scale=0.0) -> ()");
     m.def("reduce_rms_local(Tensor[] partials, Tensor residual_in, Tensor rms_gamma, Tensor residual_out, "
-          "Tensor? norm_out, Tensor? q_out, Tensor? scale_out, float eps, int quant_mode, int algo, Tensor? stage) -> ()");
+          "Tensor? norm_out, Tensor? q_out, Tensor? scale_out, float eps, int quant_mode, int algo, Tensor? stage, "
+          "float static_scale=0.0) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(torch_dist_ext, CUDA, m) {
