@@ -473,33 +473,54 @@ __global__ void __launch_bounds__(1024 / VPT)
 }
 
 // Stage A of the staged algorithm: s = T(sum of partials) for every element, no row structure.
+// One workgroup of 256 threads reduces a contiguous span of 256*U vectors (U vectors per thread,
+// all N*U loads in flight before the first add) and exits; spans past the end are cut by the buffer
+// resource's size, so there is no loop and no tail branch.
+template <int N>
+struct ReduceUnroll {
+    static constexpr int U = (N >= 8) ? 2 : 4;
+};
+
 template <class E, int N>
-__global__ void __launch_bounds__(256) reduce_kernel(const RowArgs a, int64_t total_vecs) {
+__global__ void __launch_bounds__(256) reduce_kernel(const RowArgs a, int64_t total_bytes) {
     constexpr int VEC = E::VEC;
+    constexpr int U = ReduceUnroll<N>::U;
+    constexpr uint32_t SPAN = 256u * U * 16u; // bytes per workgroup
     const void *part[N];
 #pragma unroll
-    for (int r = 0; r < N; ++r) {
-        part[r] = a.part[r];
-        if (part[r] == nullptr) part[r] = a.table[r];
-    }
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < total_vecs; v += stride) {
-        u32x4 raw[N];
+    for (int r = 0; r < N; ++r) part[r] = a.part[r];
+    if (a.table != nullptr) {
 #pragma unroll
-        for (int r = 0; r < N; ++r)
-            raw[r] = __builtin_nontemporal_load((const TDE_GLOBAL u32x4 *)((const TDE_GLOBAL char *)part[r] + v * 16));
+        for (int r = 0; r < N; ++r) {
+            const void *from_table = a.table[r];
+            part[r] = (part[r] != nullptr) ? part[r] : from_table;
+        }
+    }
+    const int64_t base = (int64_t)blockIdx.x * SPAN;
+    const int64_t left = total_bytes - base;
+    const uint32_t bytes = left < (int64_t)SPAN ? (uint32_t)left : SPAN;
+    u32x4 raw[U][N];
+#pragma unroll
+    for (int r = 0; r < N; ++r) {
+        const rsrc_t rs = row_rsrc(part[r], base, bytes);
+#pragma unroll
+        for (int u = 0; u < U; ++u) raw[u][r] = rsrc_load16(rs, (uint32_t)(u * 256 + threadIdx.x) * 16u);
+    }
+    const rsrc_t out = row_rsrc(a.stage_out, base, bytes);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
         float acc[VEC];
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
 #pragma unroll
         for (int r = 0; r < N; ++r) {
             float p[VEC];
-            E::unpack(raw[r], p);
+            E::unpack(raw[u][r], p);
 #pragma unroll
             for (int i = 0; i < VEC; ++i) acc[i] += p[i];
         }
-        // The staged sum is re-read by stage B right away: ordinary (cacheable) store.
-        *(TDE_GLOBAL u32x4 *)((TDE_GLOBAL char *)a.stage_out + v * 16) = E::pack(acc);
+        // The staged sum is re-read by stage B right away: default (cacheable) store.
+        __builtin_amdgcn_raw_buffer_store_b128(E::pack(acc), out, (int)((u * 256 + threadIdx.x) * 16), 0, kAuxDefault);
     }
 }
 
@@ -569,15 +590,14 @@ hipError_t launch_rows_e(int n, int vpt, int q, bool wn, const RowArgs &a, const
 template <class E>
 hipError_t launch_reduce_e(int n, const RowArgs &a, int64_t total_vecs, hipStream_t s) {
     if (total_vecs <= 0) return hipSuccess;
-    const int block = 256;
-    int64_t blocks = (total_vecs + block - 1) / block;
-    const int64_t cap = 256 * 16; // 16 workgroups of 4 wavefronts per CU, grid-stride beyond that
-    if (blocks > cap) blocks = cap;
-    const dim3 grid((unsigned)blocks), blk(block);
+    const int64_t total_bytes = total_vecs * 16;
+    if ((total_vecs + 511) / 512 > 0x7fffffff) return hipErrorInvalidValue; // grid dimension limit
+    auto blocks_for = [&](int u) { return (unsigned)((total_vecs + 256 * u - 1) / (256 * u)); };
+    const dim3 blk(256);
     switch (n) {
-    case 2: hipLaunchKernelGGL((reduce_kernel<E, 2>), grid, blk, 0, s, a, total_vecs); break;
-    case 4: hipLaunchKernelGGL((reduce_kernel<E, 4>), grid, blk, 0, s, a, total_vecs); break;
-    case 8: hipLaunchKernelGGL((reduce_kernel<E, 8>), grid, blk, 0, s, a, total_vecs); break;
+    case 2: hipLaunchKernelGGL((reduce_kernel<E, 2>), dim3(blocks_for(ReduceUnroll<2>::U)), blk, 0, s, a, total_bytes); break;
+    case 4: hipLaunchKernelGGL((reduce_kernel<E, 4>), dim3(blocks_for(ReduceUnroll<4>::U)), blk, 0, s, a, total_bytes); break;
+    case 8: hipLaunchKernelGGL((reduce_kernel<E, 8>), dim3(blocks_for(ReduceUnroll<8>::U)), blk, 0, s, a, total_bytes); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
