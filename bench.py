@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
 """Headline benchmark: one rank's 8-partial reduce + residual + RMSNorm + per-token fp8 quant stage
-at 2048 x 8192 bf16 (BASELINE config c3) on ONE MI355X, through the C ABI (tde_reduce_rms).
+at 2048 x 8192 bf16 (the headline configuration, here called c3) on ONE MI355X, through the C ABI (tde_reduce_rms).
 
 A step is one launch of the fused row kernel over one batch of synthetic inputs that already sit
 in HBM.  Inputs rotate over several distinct sets (> 1 GiB in total) so that no launch finds its

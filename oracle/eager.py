@@ -131,7 +131,7 @@ def make_inputs(N, T, H, dtype, sigma=1.0, seed=0, outlier_channels=0, outlier_s
 
 
 def make_config(name, tokens=None):
-    """Inputs of a named BASELINE config.  "c5" needs tokens in C5_TOKENS.  Returns
+    """Inputs of a named benchmark configuration (c1..c5).  "c5" needs tokens in C5_TOKENS.  Returns
     (parts, residual, gamma, eps, quant)."""
     if name == "c5":
         assert tokens is not None

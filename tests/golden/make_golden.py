@@ -1,5 +1,5 @@
 """Writes tests/golden/golden.npz: inputs and expected outputs of the CPU oracle (oracle/eager.py)
-for BASELINE config c1 (seed 0) and three tiny quant cases.  The reference has no golden vectors and
+for configuration c1 (2 partials, 16 x 1024 bf16, seed 0) and three tiny quant cases.  The reference has no golden vectors and
 its package is not imported here: these fixtures freeze this build's oracle so that a later change
 to it (or a different torch CPU build) is noticed.  bf16/fp16 arrays are stored as uint16 bits.
 

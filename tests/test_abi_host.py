@@ -68,7 +68,7 @@ def test_plan_null_pointers():
 
 
 @pytest.mark.parametrize("cfg,expected", [
-    # BASELINE configs: bytes = (N+1)*T*H*e + H*e + T*H*e + OUT
+    # the five benchmark configurations: bytes = (N+1)*T*H*e + H*e + T*H*e + OUT
     (dict(nranks=2, tokens=16, hidden=1024, quant=_capi.QUANT_NONE), 165888),
     (dict(nranks=8, tokens=128, hidden=4096, quant=_capi.QUANT_NONE), 11542528),
     (dict(nranks=8, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_TOKEN), 352346112),

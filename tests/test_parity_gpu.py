@@ -160,7 +160,7 @@ def test_every_launch_geometry_agrees(cuda_device, vpt, prefetch, grid):
 
 
 def test_full_size_c3_properties(cuda_device):
-    """BASELINE c3 at full size on the device only (the CPU oracle is not run at this size here):
+    """Configuration c3 at full size on the device only (the CPU oracle is not run at this size here):
     size-independent properties of the outputs."""
     dev = cuda_device
     gen = torch.Generator(device=dev).manual_seed(3)
@@ -225,7 +225,7 @@ def _device_residual(parts, res):
     ("c5@32768", 4, 32768, 5120, torch.float16, 1.0, 1e-6, "int8_token", 5),
 ])
 def test_full_size_c4_c5_properties(cuda_device, name, n, t, h, dtype, sigma, eps, quant, outliers):
-    """BASELINE c4 and the largest c5 at full size.  Inputs are drawn on the device; the residual is checked
+    """Configurations c4 and the largest c5 at full size.  Inputs are drawn on the device; the residual is checked
     against the same rank-order sum written with torch device ops, and the quant epilogue against the oracle's
     quantizer applied on the host to a band of the written normed rows (the whole tensor for the scales)."""
     import torch_dist_ext_amd as tde
