@@ -189,11 +189,12 @@ __device__ __forceinline__ const TDE_GLOBAL V *global_ptr(const void *base, uint
 // filled wavefronts nor tail rows need a branch.
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 constexpr int kRsrcFlags = 0x00020000; // raw buffer, 32-bit data format (gfx9 family encoding)
-constexpr int kAuxStream = 2;          // loads, nt: streamed once, do not keep in cache (7.0 vs 6.4 TB/s read ceiling)
-#ifndef TDE_AUX_STORE
-#define TDE_AUX_STORE 16
-#endif
-constexpr int kAuxStore = TDE_AUX_STORE; // stores, sc1: measured best for the mixed 6:1 read/write stream (nt stores cost ~8 %)
+constexpr int kAuxStream = 2; // nt on loads and stores: streamed once, do not keep in cache.
+// Measured on MI355X with inputs and outputs rotated far beyond the 256 MB memory-side cache:
+// nt loads 7.0 vs 6.4 TB/s read ceiling; nt stores 1-2 % faster than sc1 and 8 % faster than the
+// default policy on the 6:1 read/write mix.  (With outputs small enough to stay in that cache,
+// sc1 stores measure faster; that is not the HBM-bound case.)
+constexpr int kAuxStore = 2;
 constexpr int kAuxDefault = 0;
 
 __device__ __forceinline__ rsrc_t row_rsrc(const void *base, int64_t byte_off, uint32_t bytes) {
