@@ -329,3 +329,13 @@ def test_hip_graph_replays_match_eager(cuda_device):
         assert bits_equal(outs["res_out"].cpu(), got["residual_out"]) and bits_equal(outs["norm"].cpu(), got["norm_out"])
         assert bits_equal(q.cpu(), got["q"].view(torch.uint8)) and bits_equal(sc.cpu(), got["scale"])
         check_against_oracle(got, eager.reduce_rms(cp, cr, cg, 1e-5, "fp8_token"), "fp8_token", gamma=cg, eps=1e-5)
+
+
+@pytest.mark.parametrize("quant", ["none", "fp8_token", "fp8_group", "int8_token"])
+@pytest.mark.parametrize("dtype,hidden", [(torch.float16, 8192), (torch.float32, 4096), (torch.bfloat16, 6144), (torch.float32, 3072)])
+def test_long_rows_every_dtype(cuda_device, dtype, hidden, quant):
+    """Rows of 768..1024 vectors take the 4-vectors-per-thread kernels; cover them for every dtype and mode."""
+    p, r, g = eager.make_inputs(4, 19, hidden, dtype, 1.0, seed=hidden + 3)
+    assert _capi.plan(_capi.make_problem({torch.float16: _capi.F16, torch.float32: _capi.F32, torch.bfloat16: _capi.BF16}[dtype],
+                                         4, 19, hidden, 1e-6)).vecs_per_thread == 4
+    _case("long-rows", p, r, g, 1e-6, quant)

@@ -321,6 +321,11 @@ __global__ void __launch_bounds__(1024 / VPT)
     RowLoads<NP, VPT> cur;
     issue_loads(cur, row0 + group);
     const rsrc_t gamma_rsrc = row_rsrc(a.gamma, 0, row_bytes);
+    u32x4 gamma_early = u32x4{0, 0, 0, 0};
+    if constexpr (VPT == 1) {
+        __builtin_amdgcn_sched_barrier(0);
+        gamma_early = __builtin_amdgcn_raw_buffer_load_b128(gamma_rsrc, (int)lane_off[0], 0, kAuxDefault);
+    }
 
     int parity = 0;
     for (; row0 < a.tokens; row0 += row_stride, parity ^= 1) {
@@ -368,13 +373,19 @@ __global__ void __launch_bounds__(1024 / VPT)
                 else sumsq += x[i] * x[i];
             }
         }
-        // gamma (shared by all rows, served from L2) is requested only now: the registers of the row
-        // loads are free again, and the reduction below covers its latency.
-        __builtin_amdgcn_sched_barrier(0);
+        // gamma (shared by all rows, served from L2).  With several vectors per thread it is requested
+        // only now: the registers of the row loads are free again, and the reduction below covers its
+        // latency.  With one vector per thread registers are plentiful and it was requested right
+        // behind the row loads (shortest dependent chain for small, latency-bound inputs).
         u32x4 gamma_raw[VPT];
+        if constexpr (VPT > 1) {
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int j = 0; j < VPT; ++j)
-            gamma_raw[j] = __builtin_amdgcn_raw_buffer_load_b128(gamma_rsrc, (int)lane_off[j], 0, kAuxDefault);
+            for (int j = 0; j < VPT; ++j)
+                gamma_raw[j] = __builtin_amdgcn_raw_buffer_load_b128(gamma_rsrc, (int)lane_off[j], 0, kAuxDefault);
+        } else {
+            gamma_raw[0] = gamma_early;
+        }
         sumsq = row_reduce<OpSum>(sumsq, lds_sum[parity], wave, lane, first_wave, waves_per_row);
         const float rs = 1.0f / __builtin_sqrtf(sumsq / a.hidden_f + a.eps);
 
