@@ -83,9 +83,27 @@ def build_torch(verbose=False):
     return TORCH_LIB
 
 
+def build_native_test(verbose=False):
+    """tests/native/unit_test_abi: a C++ program that drives the C ABI without Python or torch and checks
+    it against the oracle's C restatement (linked in as the checker)."""
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    src = os.path.join(ROOT, "tests", "native", "unit_test_abi.cpp")
+    out = os.path.join(ROOT, "tests", "native", "unit_test_abi")
+    oracle_dir = os.path.join(ROOT, "oracle")
+    _run(["make", "-C", oracle_dir, "libtde_oracle.so"])
+    cmd = [hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", "-I", INCLUDE, src, "-o", out,
+           "-L", PKG_DIR, "-ltde_hip", "-L", oracle_dir, "-ltde_oracle",
+           "-Wl,-rpath,$ORIGIN/../../torch_dist_ext_amd", "-Wl,-rpath,$ORIGIN/../../oracle"]
+    o = _run(cmd)
+    if verbose and o.strip():
+        print(o)
+    return out
+
+
 def build_all(verbose=False):
     build_hip(verbose)
     build_torch(verbose)
+    build_native_test(verbose)
     return HIP_LIB, TORCH_LIB
 
 
