@@ -138,12 +138,11 @@ int tde_plan(const tde_problem *problem, tde_plan_out *plan);
    (impl.h:500-535) for the arithmetic of one rank; quant outputs extend it. */
 int tde_reduce_rms(const tde_problem *problem, const tde_buffers *buffers, void *hip_stream);
 
-/* Tuning hook for sweeps and tests: force vectors-per-thread (1,2), rows per workgroup, a cap on
-   the grid (rows beyond it are covered by a grid-stride loop) and the software pipeline
-   (1 = off, 2 = on).  0 restores the automatic choice for that field.  Process-wide, not
-   thread-safe.  No counterpart in the reference, whose launcher hard-codes its geometry
-   (impl.h:481-489). */
-int tde_tune_override(int32_t vecs_per_thread, int32_t rows_per_block, int32_t max_grid, int32_t prefetch);
+/* Tuning hook for sweeps and tests: force vectors-per-thread (1,2,4), rows per workgroup and a cap
+   on the grid (rows beyond it are covered by a grid-stride loop).  0 restores the automatic choice
+   for that field.  Process-wide, not thread-safe.  No counterpart in the reference, whose
+   launcher hard-codes its geometry (impl.h:481-489). */
+int tde_tune_override(int32_t vecs_per_thread, int32_t rows_per_block, int32_t max_grid);
 
 /* Calibration: enqueue a plain copy of `bytes` (multiple of 16) from src to dst on `hip_stream`.
    Known traffic (bytes read + bytes written) for scaling profiler memory counters and for

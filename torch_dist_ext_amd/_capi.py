@@ -74,7 +74,7 @@ def load():
     lib.tde_reduce_rms.restype = ctypes.c_int
     lib.tde_reduce_rms.argtypes = [ctypes.POINTER(Problem), ctypes.POINTER(Buffers), ctypes.c_void_p]
     lib.tde_tune_override.restype = ctypes.c_int
-    lib.tde_tune_override.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
+    lib.tde_tune_override.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
     lib.tde_probe_copy.restype = ctypes.c_int
     lib.tde_probe_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
     lib.tde_workspace_create.restype = ctypes.c_int
@@ -133,8 +133,8 @@ def reduce_rms(problem, partials, residual_in, residual_out, gamma, norm_out=Non
     check(load().tde_reduce_rms(ctypes.byref(problem), ctypes.byref(b), stream))
 
 
-def tune_override(vecs_per_thread=0, rows_per_block=0, max_grid=0, prefetch=0):
-    check(load().tde_tune_override(vecs_per_thread, rows_per_block, max_grid, prefetch))
+def tune_override(vecs_per_thread=0, rows_per_block=0, max_grid=0):
+    check(load().tde_tune_override(vecs_per_thread, rows_per_block, max_grid))
 
 
 def probe_copy(dst, src, nbytes, stream=None):

@@ -35,7 +35,6 @@ constexpr int kMaxBlock = 1024;
 int g_force_vpt = 0;
 int g_force_rows_per_block = 0;
 int g_force_grid = 0;
-int g_force_prefetch = 0; // 0 auto, 1 off, 2 on
 
 constexpr int kComputeUnits = 256; // MI355X
 
@@ -68,10 +67,6 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     if (g_force_rows_per_block > 0 && g_force_rows_per_block * tpr <= kMaxBlock / vpt) rpb = g_force_rows_per_block;
     if (p->tokens > 0 && rpb > p->tokens) rpb = (int)p->tokens;
     int64_t grid = (p->tokens + rpb - 1) / rpb;
-    // Software-pipelined persistent launch once there are several rows per compute unit: one
-    // resident workgroup set, each workgroup walking its rows with the next row's loads in flight.
-    bool prefetch = false;
-    if (g_force_prefetch == 2) prefetch = true;
     if (g_force_grid > 0 && grid > g_force_grid) grid = g_force_grid;
     if (grid > 0x7fffffff) return TDE_ESHAPE;
 
@@ -83,7 +78,6 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
         geo->rows_per_block = rpb;
         geo->block_threads = tpr * rpb;
         geo->grid = grid;
-        geo->prefetch = prefetch;
     }
     return TDE_OK;
 }
@@ -149,11 +143,10 @@ const char *tde_status_string(int status) {
 
 int tde_last_hip_error(void) { return g_last_hip_error; }
 
-int tde_tune_override(int32_t vecs_per_thread, int32_t rows_per_block, int32_t max_grid, int32_t prefetch) {
+int tde_tune_override(int32_t vecs_per_thread, int32_t rows_per_block, int32_t max_grid) {
     g_force_vpt = vecs_per_thread;
     g_force_rows_per_block = rows_per_block;
     g_force_grid = max_grid;
-    g_force_prefetch = prefetch;
     return TDE_OK;
 }
 

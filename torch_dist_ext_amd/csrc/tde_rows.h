@@ -260,14 +260,12 @@ struct RowLoads {
 //   VPT    16-byte vectors per thread per row (1 or 2)
 //   Q      tde_quant
 //   WN     write the T-typed normed row (always true for Q == NONE)
-//   PF     software pipeline: the loads of the block's next row are issued before the current row is
-//          consumed, so a workgroup always has a full row of requests in flight
 // Block layout: rows_per_block row groups of threads_per_row threads; thread t of a row group
 // owns vectors t, t + threads_per_row, ... (coalesced 1 KiB per wavefront per load).
 // ---------------------------------------------------------------------------------------------
-template <class E, int N, int VPT, int Q, bool WN, bool PF>
+template <class E, int N, int VPT, int Q, bool WN>
 __global__ void __launch_bounds__(1024 / VPT)
-    __attribute__((amdgpu_waves_per_eu(PF ? 4 : (VPT == 1 ? 8 : (VPT == 2 ? 5 : 3))))) row_kernel(const RowArgs a) {
+    __attribute__((amdgpu_waves_per_eu(VPT == 1 ? 8 : (VPT == 2 ? 5 : 3)))) row_kernel(const RowArgs a) {
     constexpr int VEC = E::VEC;
     constexpr int NP = (N == 0) ? 1 : N;
     __shared__ float lds_sum[2][kMaxWavesPerBlock];
@@ -333,9 +331,6 @@ __global__ void __launch_bounds__(1024 / VPT)
         const bool row_ok = row < a.tokens;
         const uint32_t bytes = row_ok ? row_bytes : 0u;
         const int64_t row_byte = row * (int64_t)row_bytes; // wavefront-uniform
-
-        RowLoads<NP, VPT> nxt;
-        if constexpr (PF) issue_loads(nxt, row + row_stride); // past-the-end rows load nothing
 
         // ---- reduce, residual add, sum of squares ------------------------------------------------
         const rsrc_t res_out = row_rsrc(a.residual_out, row_byte, bytes);
@@ -476,11 +471,8 @@ __global__ void __launch_bounds__(1024 / VPT)
                 }
             }
         }
-        if constexpr (PF) {
-            cur = nxt;
-        } else {
-            if (row0 + row_stride < a.tokens) issue_loads(cur, row + row_stride);
-        }
+        // Only a capped grid comes round again; the next row's loads go out behind this row's stores.
+        if (row0 + row_stride < a.tokens) issue_loads(cur, row + row_stride);
     }
 }
 
@@ -547,7 +539,6 @@ struct Geometry {
     int rows_per_block;
     int block_threads;
     int64_t grid;
-    bool prefetch;
 };
 
 // Per-dtype launchers, defined in tde_rows_<dtype>.hip.
@@ -559,11 +550,11 @@ hipError_t launch_reduce_f16(int n, const RowArgs &a, int64_t total_vecs, hipStr
 hipError_t launch_reduce_f32(int n, const RowArgs &a, int64_t total_vecs, hipStream_t s);
 
 // Instantiation + dispatch body used by the three per-dtype translation units.
-template <class E, int N, int VPT, bool PF>
-hipError_t launch_rows_nvp(int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s) {
+template <class E, int N, int VPT>
+hipError_t launch_rows_nv(int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s) {
     const dim3 grid((unsigned)g.grid), block((unsigned)g.block_threads);
 #define TDE_LAUNCH(QM, WNB)                                                       \
-    hipLaunchKernelGGL((row_kernel<E, N, VPT, QM, WNB, PF>), grid, block, 0, s, a); \
+    hipLaunchKernelGGL((row_kernel<E, N, VPT, QM, WNB>), grid, block, 0, s, a); \
     return hipGetLastError();
     switch (q) {
     case TDE_QUANT_NONE: TDE_LAUNCH(TDE_QUANT_NONE, true)
@@ -582,9 +573,9 @@ hipError_t launch_rows_nvp(int q, bool wn, const RowArgs &a, const Geometry &g, 
 
 template <class E, int N>
 hipError_t launch_rows_n(int vpt, int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s) {
-    if (vpt == 1) return g.prefetch ? launch_rows_nvp<E, N, 1, true>(q, wn, a, g, s) : launch_rows_nvp<E, N, 1, false>(q, wn, a, g, s);
-    if (vpt == 2) return launch_rows_nvp<E, N, 2, false>(q, wn, a, g, s);
-    if (vpt == 4) return launch_rows_nvp<E, N, 4, false>(q, wn, a, g, s);
+    if (vpt == 1) return launch_rows_nv<E, N, 1>(q, wn, a, g, s);
+    if (vpt == 2) return launch_rows_nv<E, N, 2>(q, wn, a, g, s);
+    if (vpt == 4) return launch_rows_nv<E, N, 4>(q, wn, a, g, s);
     return hipErrorInvalidValue;
 }
 
