@@ -173,15 +173,9 @@ __device__ __forceinline__ float row_reduce(float v, float *slots, int wave, int
     return row16_reduce<Op>(t);
 }
 
-// Streaming (non-temporal) 128-bit access at a wavefront-uniform base plus a 32-bit lane offset:
-// the form that maps to global_load/store_dwordx4 with an SGPR base.
-// Every buffer is device (global) memory, so plain accesses are typed as address space 1 and never
-// go through the flat aperture check.
+// Every buffer is device (global) memory: the few accesses that do not go through a buffer resource
+// are typed as address space 1, so they never take the flat aperture check.
 #define TDE_GLOBAL __attribute__((address_space(1)))
-template <class V>
-__device__ __forceinline__ const TDE_GLOBAL V *global_ptr(const void *base, uint32_t byte_off) {
-    return (const TDE_GLOBAL V *)((const TDE_GLOBAL char *)base + byte_off);
-}
 
 // Row-sized buffer resources.  A row is addressed as (wavefront-uniform 128-bit resource in SGPRs)
 // + (32-bit lane offset in one VGPR).  The resource's size is the row's byte length, or 0 for a row
@@ -257,7 +251,7 @@ struct RowLoads {
 //   E      element traits
 //   N      number of partials summed per element; N == 0 means "the sum was staged":
 //          part[0] already holds s (a T-typed [tokens,hidden] buffer)
-//   VPT    16-byte vectors per thread per row (1 or 2)
+//   VPT    16-byte vectors per thread per row (1, 2 or 4)
 //   Q      tde_quant
 //   WN     write the T-typed normed row (always true for Q == NONE)
 // Block layout: rows_per_block row groups of threads_per_row threads; thread t of a row group
