@@ -331,10 +331,16 @@ def test_hip_graph_replays_match_eager(cuda_device):
 
 
 @pytest.mark.parametrize("quant", ["none", "fp8_token", "fp8_group", "int8_token"])
-@pytest.mark.parametrize("dtype,hidden", [(torch.float16, 8192), (torch.float32, 4096), (torch.bfloat16, 6144), (torch.float32, 3072)])
+@pytest.mark.parametrize("dtype,hidden", [(torch.float16, 8192), (torch.float32, 4096), (torch.bfloat16, 7168), (torch.float32, 3584)])
 def test_long_rows_every_dtype(cuda_device, dtype, hidden, quant):
-    """Rows of 768..1024 vectors take the 4-vectors-per-thread kernels; cover them for every dtype and mode."""
+    """Rows of 896..1024 vectors take the 4-vectors-per-thread kernels once there are many rows; cover them
+    for every dtype and mode (forced here, the input has few rows)."""
     p, r, g = eager.make_inputs(4, 19, hidden, dtype, 1.0, seed=hidden + 3)
-    assert _capi.plan(_capi.make_problem({torch.float16: _capi.F16, torch.float32: _capi.F32, torch.bfloat16: _capi.BF16}[dtype],
-                                         4, 19, hidden, 1e-6)).vecs_per_thread == 4
-    _case("long-rows", p, r, g, 1e-6, quant)
+    code = {torch.float16: _capi.F16, torch.float32: _capi.F32, torch.bfloat16: _capi.BF16}[dtype]
+    assert _capi.plan(_capi.make_problem(code, 4, 4096, hidden, 1e-6)).vecs_per_thread == 4
+    assert _capi.plan(_capi.make_problem(code, 4, 19, hidden, 1e-6)).vecs_per_thread == 1
+    _capi.tune_override(4, 0, 0)
+    try:
+        _case("long-rows", p, r, g, 1e-6, quant)
+    finally:
+        _capi.tune_override(0, 0, 0)

@@ -55,14 +55,21 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     if (nvec > kMaxBlock) return TDE_EHIDDEN; // as the reference: one 16-byte vector per thread, 1024 threads
     if (p->tokens > 0 && p->tokens * p->hidden / p->hidden != p->tokens) return TDE_ESHAPE;
 
-    // Vectors per thread: long rows use small workgroups that each keep many loads in flight
-    // (measured best on MI355X: 256-thread groups with 4 vectors per thread at 1024 vectors per row).
-    int vpt = (nvec >= 768) ? 4 : 1;
+    // Vectors per thread.  Four vectors per thread (small workgroups, many loads in flight per thread,
+    // few wavefronts to synchronize per row) win where they fill their lanes: rows of 896+ vectors, and
+    // rows of exactly 256/512/1024 vectors (one, two or four full wavefronts per row); measured on
+    // MI355X across hidden 2048..8192, the other sizes are as fast or faster with one vector per thread,
+    // as are 512-vector rows with four or fewer partials.
+    int vpt = 1;
+    if (nvec >= 896) vpt = 4;
+    else if (nvec == 256 || (nvec == 512 && p->nranks >= 8)) vpt = 4;
+    if (p->tokens < 1024) vpt = 1; // few rows: latency-bound, the widest row groups have the shortest chain
     if (g_force_vpt == 1 || g_force_vpt == 2 || g_force_vpt == 4) vpt = g_force_vpt;
     const int64_t lanes = (nvec + vpt - 1) / vpt;
     const int tpr = (int)((lanes + 63) / 64 * 64);
     int rpb = 256 / tpr; // pack short rows so a workgroup has at least four wavefronts
     if (rpb * tpr > kMaxBlock / vpt) rpb = (kMaxBlock / vpt) / tpr; // never beyond the kernel's launch bound
+    while (rpb > 1 && (p->tokens + rpb - 1) / rpb < 2 * kComputeUnits) rpb /= 2; // keep every CU busy first
     if (rpb < 1) rpb = 1;
     if (g_force_rows_per_block > 0 && g_force_rows_per_block * tpr <= kMaxBlock / vpt) rpb = g_force_rows_per_block;
     if (p->tokens > 0 && rpb > p->tokens) rpb = (int)p->tokens;
