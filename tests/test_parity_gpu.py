@@ -344,3 +344,59 @@ def test_long_rows_every_dtype(cuda_device, dtype, hidden, quant):
         _case("long-rows", p, r, g, 1e-6, quant)
     finally:
         _capi.tune_override(0, 0, 0)
+
+
+def test_randomized_shapes_and_modes(cuda_device):
+    """Seeded sweep over random (dtype, N, tokens, hidden, mode) combinations, small enough for the CPU oracle:
+    exercises row packing, partly filled wavefronts and every kernel family in one go."""
+    rng = torch.Generator().manual_seed(2024)
+    dtypes = [torch.bfloat16, torch.float16, torch.float32]
+    modes = ["none", "fp8_token", "fp8_group", "int8_token"]
+    done = 0
+    for _ in range(64):
+        dtype = dtypes[int(torch.randint(0, 3, (1,), generator=rng))]
+        n = [2, 4, 8][int(torch.randint(0, 3, (1,), generator=rng))]
+        tokens = int(torch.randint(1, 70, (1,), generator=rng))
+        vec = 4 if dtype == torch.float32 else 8
+        nvec = int(torch.randint(1, 1025, (1,), generator=rng))
+        quant = modes[int(torch.randint(0, 4, (1,), generator=rng))]
+        hidden = nvec * vec
+        if quant == "fp8_group":
+            hidden = max(128, hidden // 128 * 128)
+        p, r, g = eager.make_inputs(n, tokens, hidden, dtype, 1.0, seed=1000 + done)
+        _case("fuzz%d" % done, p, r, g, 1e-6, quant)
+        done += 1
+    assert done == 64
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("scale", [1e-30, 3e-39, 1e-6, 1e4])
+def test_extreme_magnitudes(cuda_device, dtype, scale):
+    """Very small (down to fp32 subnormals) and large inputs: the reduce and the residual add stay bit-exact,
+    i.e. the kernel neither flushes subnormals nor rounds differently near the ends of the range."""
+    if dtype == torch.float16 and scale < 1e-6:
+        scale = 6e-8 * (1 if scale < 1e-30 else 40)     # fp16 subnormal range
+    if dtype == torch.float16 and scale > 100:
+        scale = 2000.0                                    # sums reach past 65504: rounds to inf in both
+    p, r, g = eager.make_inputs(4, 9, 512, torch.float32, 1.0, seed=61)
+    p, r = (p * scale).to(dtype), (r * scale).to(dtype)
+    g = g.to(dtype)
+    want = eager.reduce_rms(p, r, g, 1e-6)
+    got = run_hip(p, r, g, 1e-6, "none")
+    assert bits_equal(got["residual_out"], want["residual_out"])
+    finite = torch.isfinite(want["norm_out"].float()) & torch.isfinite(got["norm_out"].float())
+    assert bool((torch.isfinite(want["norm_out"].float()) == torch.isfinite(got["norm_out"].float())).all())
+    from helpers import ulp_distance as _ud
+    d = _ud(got["norm_out"], want["norm_out"])[finite]
+    assert d.numel() == 0 or int(d.max()) <= (8 if dtype == torch.float32 else 2)
+
+
+@pytest.mark.parametrize("quant", ["fp8_token", "fp8_group", "int8_token"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("gscale", [1e-30, 1e25])
+def test_quant_with_scales_outside_the_fast_division_range(cuda_device, dtype, quant, gscale):
+    """gamma of 1e-30 / 1e25 pushes the dynamic scale below 2^-60 / above 2^60, where the kernel leaves its
+    reciprocal-based quotient for a plain division: codes and scales must still be the oracle's, bit for bit."""
+    p, r, g = eager.make_inputs(4, 11, 1024, torch.float32, 1.0, seed=71)
+    p, r, g = p.to(dtype), r.to(dtype), (g * gscale).to(dtype)
+    _case("tiny-scale", p, r, g, 1e-6, quant)
