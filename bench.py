@@ -87,7 +87,7 @@ def main():
     ap.add_argument("--config", default="c3", choices=sorted(BENCH_CONFIGS))
     ap.add_argument("--sets", type=int, default=0, help="distinct input sets to rotate over (0 = enough for > 1 GiB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--algo", default="auto", choices=["auto", "fused", "staged"])
+    ap.add_argument("--algo", default="auto", choices=["auto", "fused", "staged", "staged_owned"])
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (one rank's stage with N local partial buffers); "
@@ -106,7 +106,8 @@ def main():
     N, T, H, dt, sigma, eps, quant = cfg
     qm = {"none": _capi.QUANT_NONE, "fp8_token": _capi.QUANT_FP8_TOKEN, "fp8_group": _capi.QUANT_FP8_GROUP,
           "int8_token": _capi.QUANT_INT8_TOKEN}[quant]
-    algo = {"auto": _capi.ALGO_AUTO, "fused": _capi.ALGO_FUSED, "staged": _capi.ALGO_STAGED}[args.algo]
+    algo = {"auto": _capi.ALGO_AUTO, "fused": _capi.ALGO_FUSED, "staged": _capi.ALGO_STAGED,
+            "staged_owned": _capi.ALGO_STAGED_OWNED}[args.algo]
     dcode = {"bf16": _capi.BF16, "f16": _capi.F16, "f32": _capi.F32}[dt]
     prob = _capi.make_problem(dcode, N, T, H, eps, quant=qm, algo=algo, write_norm=0)
     plan = _capi.plan(prob)
@@ -118,7 +119,16 @@ def main():
     out_bytes = bytes_per_launch - (N + 1) * T * H * e - H * e
     nsets = args.sets or min(128, max(3, -(-(4 << 30) // bytes_per_launch), -(-(1 << 30) // max(out_bytes, 1))) + 1)
     sets, gamma, dtype = make_sets(torch, cfg, nsets, dev)
-    stage = torch.empty((T, H), dtype=dtype, device=dev) if algo == _capi.ALGO_STAGED else None
+    staged = algo in (_capi.ALGO_STAGED, _capi.ALGO_STAGED_OWNED)
+    # One stage buffer per input set, so that stage B reads it from HBM like everything else.
+    stages = [torch.zeros((T, H), dtype=dtype, device=dev) for _ in range(nsets)] if staged else None
+    if algo == _capi.ALGO_STAGED_OWNED:
+        # One rank's local share of the two-shot: stage A touches T/N rows of the N partials, stage B all T rows
+        # of the stage (the rows of the other ranks are taken as already delivered; they are zeros here).
+        owned = -(-T // N)
+        bytes_per_launch = (N + 1) * owned * H * e + 2 * T * H * e + H * e + T * H * e + out_bytes
+    elif staged:
+        bytes_per_launch += 2 * T * H * e      # the stage is written once and read once on top of the fused job
     stream = torch.cuda.current_stream(dev)
 
     # Argument blocks are built once per input set; a step is then a single C-ABI call.
@@ -133,7 +143,7 @@ def main():
         b.norm_out = s["norm"].data_ptr() if s["norm"] is not None else None
         b.q_out = s["q"].data_ptr() if s["q"] is not None else None
         b.scale_out = s["scale"].data_ptr() if s["scale"] is not None else None
-        b.stage = stage.data_ptr() if stage is not None else None
+        b.stage = stages[len(calls)].data_ptr() if staged else None
         calls.append(b)
     prob_ref = ctypes.byref(prob)
     call_refs = [ctypes.byref(b) for b in calls]
@@ -184,11 +194,14 @@ def main():
         "dtype": dt, "data": "synthetic",
         "tokens_per_s": T / (wall / args.steps),
         "pct_of_hbm_peak": 100.0 * gbs_job / HBM_PEAK_GBS,
-        "config": {"workload": "%s: N=%d partials [%d,%d] %s, residual add + RMSNorm + %s" % (args.config, N, T, H, dt, quant),
+        "config": {"workload": "%s: N=%d partials [%d,%d] %s, residual add + RMSNorm + %s%s" % (
+                       args.config, N, T, H, dt, quant,
+                       {"staged": " (two launches through a stage buffer)",
+                        "staged_owned": " (two launches; stage A over this rank's T/N rows only)"}.get(args.algo, "")),
                    "algo": args.algo, "input_sets": nsets, "block_threads": plan.block_threads,
                    "grid_blocks": plan.grid_blocks, "algorithmic_bytes": bytes_per_launch},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get(args.config),
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None if staged else TRAFFIC_BYTES.get(args.config),
                      "kernel_avg_us": avg_ms * 1e3},
     }
     if not args.no_cpu_baseline:

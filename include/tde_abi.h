@@ -67,8 +67,11 @@ typedef enum tde_algo {
     TDE_ALGO_AUTO = 0,   /* = TDE_ALGO_FUSED */
     TDE_ALGO_FUSED = 1,  /* one pass per row: reduce -> residual -> norm -> quant, row kept in registers
                             (the arithmetic of the one-shot body, impl.h:450-471) */
-    TDE_ALGO_STAGED = 2  /* two launches: (A) N-way reduce of every row into `stage` (impl.h:365-377),
+    TDE_ALGO_STAGED = 2, /* two launches: (A) N-way reduce of every row into `stage` (impl.h:365-377),
                             (B) residual + norm (+quant) reading `stage` (impl.h:381-393) */
+    TDE_ALGO_STAGED_OWNED = 3 /* as STAGED, but (A) reduces only this rank's share, rows == rank (mod nranks), as one
+                            rank of the reference's two-shot does (impl.h:366); the other rows of `stage` must already
+                            hold their sums (in the reference the peers write them, impl.h:373-376) */
 } tde_algo;
 
 /* ---- problem / buffers ---------------------------------------------------------------------- */

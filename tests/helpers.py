@@ -34,9 +34,10 @@ def bits_equal(a: torch.Tensor, b: torch.Tensor) -> bool:
 
 
 def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, write_norm=None, use_table=False,
-            rank=0, device="cuda:0", static_scale=0.0):
+            rank=0, device="cuda:0", static_scale=0.0, stage_init=None):
     """Run the HIP path through the C ABI (tde_reduce_rms) on CPU inputs; returns CPU outputs.
-    parts: [N,T,H] tensor or list of N [T,H] tensors."""
+    parts: [N,T,H] tensor or list of N [T,H] tensors.  stage_init: [T,H] initial content of the stage
+    buffer (staged algorithms); the stage is then returned as out["stage"]."""
     dev = torch.device(device)
     n = len(parts)
     T, H = residual.shape
@@ -56,7 +57,11 @@ def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, wri
         nscale = T * (H // 128) if quant == "fp8_group" else T
         if quant != "fp8_static":
             d_scale = torch.empty((nscale,), dtype=torch.float32, device=dev)
-    d_stage = torch.empty_like(d_res) if algo == _capi.ALGO_STAGED else None
+    d_stage = None
+    if stage_init is not None:
+        d_stage = stage_init.contiguous().to(dev)
+    elif algo in (_capi.ALGO_STAGED, _capi.ALGO_STAGED_OWNED):
+        d_stage = torch.empty_like(d_res)
     prob = _capi.make_problem(DTYPE_CODE[dtype], n, T, H, eps, quant=qm, algo=algo, write_norm=int(bool(write_norm)),
                               rank=rank, static_scale=static_scale)
     ptrs = [p.data_ptr() for p in d_parts]
@@ -75,6 +80,8 @@ def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, wri
                      partial_table=table, stream=stream)
     torch.cuda.synchronize(dev)
     out = {"residual_out": d_res_out.cpu()}
+    if stage_init is not None:
+        out["stage"] = d_stage.cpu()
     if d_norm is not None:
         out["norm_out"] = d_norm.cpu()
     if qm:

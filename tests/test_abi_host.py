@@ -96,6 +96,7 @@ def test_plan_geometry_and_reference_threshold():
             assert q.grid_blocks * q.rows_per_block >= 777
     assert _plan(tokens=0).grid_blocks == 0
     assert _plan(algo=_capi.ALGO_STAGED).algo == _capi.ALGO_STAGED and _plan().algo == _capi.ALGO_FUSED
+    assert _plan(algo=_capi.ALGO_STAGED_OWNED).algo == _capi.ALGO_STAGED_OWNED
     assert _plan(quant=_capi.QUANT_FP8_GROUP, hidden=7168, nranks=4, tokens=8192).scale_elems == 8192 * 56
 
 

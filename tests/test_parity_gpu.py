@@ -64,6 +64,48 @@ def test_staged_equals_fused(cuda_device, quant):
         assert bits_equal(a[k], b[k]), k
 
 
+def _rank_order_sum(parts):
+    acc = torch.zeros(parts.shape[1:], dtype=torch.float32)
+    for r in range(parts.shape[0]):
+        acc = acc + parts[r].float()
+    return acc.to(parts.dtype)
+
+
+@pytest.mark.parametrize("n,rank,tokens,hidden,dtype,quant", [
+    (4, 0, 130, 2048, torch.bfloat16, "none"),
+    (4, 3, 130, 2048, torch.bfloat16, "fp8_token"),
+    (8, 5, 67, 4096, torch.bfloat16, "fp8_group"),
+    (8, 7, 3, 1024, torch.float16, "int8_token"),   # fewer rows than ranks: rank 7 owns none
+    (2, 1, 129, 1024, torch.float32, "none"),
+    (8, 2, 40, 8192, torch.bfloat16, "fp8_token"),
+    (4, 1, 33, 1000, torch.bfloat16, "none"),       # row not a multiple of the span
+])
+def test_staged_owned_rows(cuda_device, n, rank, tokens, hidden, dtype, quant):
+    """One rank of the reference's two-shot (all_reduce_fusion_impl.h:365-393): stage A sums only
+    rows == rank (mod N); the peers' rows of the stage are already there.  The owned rows start as
+    NaN, the others as the oracle's sums: the final outputs must equal the fused path bit for bit,
+    the owned rows of the stage must be the rank-order sums and the other rows must be untouched."""
+    p, r, g = eager.make_inputs(n, tokens, hidden, dtype, 1.0, seed=300 + n + rank)
+    sums = _rank_order_sum(p)
+    init = sums.clone()
+    init[rank::n] = float("nan")
+    a = run_hip(p, r, g, 1e-6, quant, algo=_capi.ALGO_FUSED, rank=rank)
+    b = run_hip(p, r, g, 1e-6, quant, algo=_capi.ALGO_STAGED_OWNED, rank=rank, stage_init=init)
+    assert bits_equal(b.pop("stage"), sums)
+    for k in a:
+        assert bits_equal(a[k], b[k]), k
+    # a wrong share is visible: with nothing pre-filled, rows of other ranks stay NaN
+    if tokens > 1:
+        c = run_hip(p, r, g, 1e-6, quant, algo=_capi.ALGO_STAGED_OWNED, rank=rank,
+                    stage_init=torch.full_like(sums, float("nan")))
+        own = torch.zeros(tokens, dtype=torch.bool)
+        own[rank::n] = True
+        assert bits_equal(c["stage"][own], sums[own])
+        assert torch.isnan(c["stage"][~own].float()).all()
+        assert bits_equal(c["residual_out"][own], a["residual_out"][own])
+        assert torch.isnan(c["residual_out"][~own].float()).all()
+
+
 def test_pointer_table_equals_direct(cuda_device):
     p, r, g = eager.make_inputs(8, 33, 4096, torch.bfloat16, 0.5, seed=22)
     a = run_hip(p, r, g, 1e-5, "fp8_token")

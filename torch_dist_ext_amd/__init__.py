@@ -18,7 +18,7 @@ from typing import Tuple
 import torch
 
 from . import _capi
-from ._capi import (ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, QUANT_FP8_GROUP, QUANT_FP8_STATIC, QUANT_FP8_TOKEN, QUANT_INT8_TOKEN,
+from ._capi import (ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, ALGO_STAGED_OWNED, QUANT_FP8_GROUP, QUANT_FP8_STATIC, QUANT_FP8_TOKEN, QUANT_INT8_TOKEN,
                     QUANT_NONE, QUANT_GROUP)
 
 this_dir = os.path.dirname(os.path.abspath(__file__))
@@ -183,7 +183,7 @@ def reduce_rms(partials, residual_in, rms_gamma, eps, quant_mode=QUANT_NONE, wri
         if quant_mode != QUANT_FP8_STATIC:
             scale_out = torch.empty(scale_shape, dtype=torch.float32, device=ref.device)
             out["scale"] = scale_out
-    if algo == ALGO_STAGED and stage is None:
+    if algo in (ALGO_STAGED, ALGO_STAGED_OWNED) and stage is None:
         stage = torch.empty_like(ref)
     reduce_rms_local_impl(list(partials), residual_in, rms_gamma, out["residual_out"], norm_out, q_out, scale_out, eps,
                           quant_mode, algo, stage, static_scale)

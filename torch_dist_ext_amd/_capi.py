@@ -13,7 +13,7 @@ QUANT_GROUP = 128
 OK, EINVAL, ENRANKS, EDTYPE, ESHAPE, EHIDDEN, EALIGN, EQUANT, EALGO, EHIP, ERANK, ENOMEM = range(12)
 BF16, F16, F32 = 0, 1, 2
 QUANT_NONE, QUANT_FP8_TOKEN, QUANT_FP8_GROUP, QUANT_INT8_TOKEN, QUANT_FP8_STATIC = 0, 1, 2, 3, 4
-ALGO_AUTO, ALGO_FUSED, ALGO_STAGED = 0, 1, 2
+ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, ALGO_STAGED_OWNED = 0, 1, 2, 3
 
 # Every symbol include/tde_abi.h declares.
 EXPORTS = (

@@ -49,7 +49,7 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     if (p->quant < TDE_QUANT_NONE || p->quant > TDE_QUANT_FP8_STATIC) return TDE_EQUANT;
     if (p->quant == TDE_QUANT_FP8_STATIC && !(p->static_scale > 0.0f && p->static_scale <= 3.0e38f)) return TDE_EQUANT;
     if (p->quant == TDE_QUANT_FP8_GROUP && p->hidden % TDE_QUANT_GROUP != 0) return TDE_EQUANT;
-    if (p->algo < TDE_ALGO_AUTO || p->algo > TDE_ALGO_STAGED) return TDE_EALGO;
+    if (p->algo < TDE_ALGO_AUTO || p->algo > TDE_ALGO_STAGED_OWNED) return TDE_EALGO;
     const int vec = 16 / eb;
     const int64_t nvec = p->hidden / vec;
     if (nvec > kMaxBlock) return TDE_EHIDDEN; // as the reference: one 16-byte vector per thread, 1024 threads
@@ -175,7 +175,7 @@ int tde_plan(const tde_problem *problem, tde_plan_out *plan) {
     const int st = validate(problem, &g);
     if (st != TDE_OK) return st;
     std::memset(plan, 0, sizeof(*plan));
-    plan->algo = (problem->algo == TDE_ALGO_STAGED) ? TDE_ALGO_STAGED : TDE_ALGO_FUSED;
+    plan->algo = (problem->algo == TDE_ALGO_STAGED || problem->algo == TDE_ALGO_STAGED_OWNED) ? problem->algo : TDE_ALGO_FUSED;
     plan->reference_algo = (problem->tokens <= 128) ? 1 : 2;
     plan->vec_elems = g.vec_elems;
     plan->block_threads = g.block_threads;
@@ -194,7 +194,7 @@ int tde_reduce_rms(const tde_problem *p, const tde_buffers *b, void *hip_stream)
     if (p->tokens == 0) return TDE_OK; // nothing to do; empty buffers may be null
     const bool quant = p->quant != TDE_QUANT_NONE;
     const bool wn = !quant || p->write_norm != 0;
-    const bool staged = p->algo == TDE_ALGO_STAGED;
+    const bool staged = p->algo == TDE_ALGO_STAGED || p->algo == TDE_ALGO_STAGED_OWNED;
 
     for (int r = 0; r < p->nranks; ++r) {
         if (b->partial[r] == nullptr && b->partial_table == nullptr) return TDE_EINVAL;
@@ -234,11 +234,19 @@ int tde_reduce_rms(const tde_problem *p, const tde_buffers *b, void *hip_stream)
     int n = p->nranks;
     hipError_t e = hipSuccess;
     if (staged) {
-        const int64_t total_vecs = p->tokens * (int64_t)g.nvec;
+        // All rows as one span of bytes, or only this rank's share (rows == rank mod nranks) row by row.
+        const int64_t row_bytes = (int64_t)g.nvec * 16;
+        int64_t span_bytes = p->tokens * row_bytes, first = 0, step = 1, rows = 1;
+        if (p->algo == TDE_ALGO_STAGED_OWNED) {
+            span_bytes = row_bytes;
+            first = p->rank;
+            step = p->nranks;
+            rows = (p->tokens - p->rank + p->nranks - 1) / p->nranks;
+        }
         switch (p->dtype) {
-        case TDE_BF16: e = tde::launch_reduce_bf16(n, a, total_vecs, stream); break;
-        case TDE_F16: e = tde::launch_reduce_f16(n, a, total_vecs, stream); break;
-        case TDE_F32: e = tde::launch_reduce_f32(n, a, total_vecs, stream); break;
+        case TDE_BF16: e = tde::launch_reduce_bf16(n, a, span_bytes, first, step, rows, stream); break;
+        case TDE_F16: e = tde::launch_reduce_f16(n, a, span_bytes, first, step, rows, stream); break;
+        case TDE_F32: e = tde::launch_reduce_f32(n, a, span_bytes, first, step, rows, stream); break;
         }
         if (e != hipSuccess) return hip_fail(e);
         for (int r = 0; r < tde::kMaxKernelRanks; ++r) a.part[r] = nullptr;

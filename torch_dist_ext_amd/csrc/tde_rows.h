@@ -479,8 +479,18 @@ struct ReduceUnroll {
     static constexpr int U = (N >= 8) ? 2 : 4;
 };
 
+// Which bytes stage A covers: `row_bytes` long rows first_row, first_row + row_step, ...; each row is cut
+// into spans_per_row spans.  The whole tensor as one long "row" (first_row 0) is the all-rows form; the
+// reference's two-shot share of one rank is rows == rank (mod nranks) (impl.h:365-366).
+struct ReduceSpan {
+    int64_t row_bytes;
+    int64_t first_row;
+    int64_t row_step;
+    int64_t spans_per_row;
+};
+
 template <class E, int N>
-__global__ void __launch_bounds__(256) reduce_kernel(const RowArgs a, int64_t total_bytes) {
+__global__ void __launch_bounds__(256) reduce_kernel(const RowArgs a, const ReduceSpan sp) {
     constexpr int VEC = E::VEC;
     constexpr int U = ReduceUnroll<N>::U;
     constexpr uint32_t SPAN = 256u * U * 16u; // bytes per workgroup
@@ -494,8 +504,10 @@ __global__ void __launch_bounds__(256) reduce_kernel(const RowArgs a, int64_t to
             part[r] = (part[r] != nullptr) ? part[r] : from_table;
         }
     }
-    const int64_t base = (int64_t)blockIdx.x * SPAN;
-    const int64_t left = total_bytes - base;
+    const int64_t k = (int64_t)blockIdx.x / sp.spans_per_row;
+    const int64_t in_row = ((int64_t)blockIdx.x - k * sp.spans_per_row) * SPAN;
+    const int64_t base = (sp.first_row + k * sp.row_step) * sp.row_bytes + in_row;
+    const int64_t left = sp.row_bytes - in_row;
     const uint32_t bytes = left < (int64_t)SPAN ? (uint32_t)left : SPAN;
     u32x4 raw[U][N];
 #pragma unroll
@@ -539,9 +551,9 @@ struct Geometry {
 hipError_t launch_rows_bf16(int n, int vpt, int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s);
 hipError_t launch_rows_f16(int n, int vpt, int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s);
 hipError_t launch_rows_f32(int n, int vpt, int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s);
-hipError_t launch_reduce_bf16(int n, const RowArgs &a, int64_t total_vecs, hipStream_t s);
-hipError_t launch_reduce_f16(int n, const RowArgs &a, int64_t total_vecs, hipStream_t s);
-hipError_t launch_reduce_f32(int n, const RowArgs &a, int64_t total_vecs, hipStream_t s);
+hipError_t launch_reduce_bf16(int n, const RowArgs &a, int64_t row_bytes, int64_t first_row, int64_t row_step, int64_t rows, hipStream_t s);
+hipError_t launch_reduce_f16(int n, const RowArgs &a, int64_t row_bytes, int64_t first_row, int64_t row_step, int64_t rows, hipStream_t s);
+hipError_t launch_reduce_f32(int n, const RowArgs &a, int64_t row_bytes, int64_t first_row, int64_t row_step, int64_t rows, hipStream_t s);
 
 // Instantiation + dispatch body used by the three per-dtype translation units.
 template <class E, int N, int VPT>
@@ -584,20 +596,28 @@ hipError_t launch_rows_e(int n, int vpt, int q, bool wn, const RowArgs &a, const
     return hipErrorInvalidValue;
 }
 
-template <class E>
-hipError_t launch_reduce_e(int n, const RowArgs &a, int64_t total_vecs, hipStream_t s) {
-    if (total_vecs <= 0) return hipSuccess;
-    const int64_t total_bytes = total_vecs * 16;
-    if ((total_vecs + 511) / 512 > 0x7fffffff) return hipErrorInvalidValue; // grid dimension limit
-    auto blocks_for = [&](int u) { return (unsigned)((total_vecs + 256 * u - 1) / (256 * u)); };
-    const dim3 blk(256);
-    switch (n) {
-    case 2: hipLaunchKernelGGL((reduce_kernel<E, 2>), dim3(blocks_for(ReduceUnroll<2>::U)), blk, 0, s, a, total_bytes); break;
-    case 4: hipLaunchKernelGGL((reduce_kernel<E, 4>), dim3(blocks_for(ReduceUnroll<4>::U)), blk, 0, s, a, total_bytes); break;
-    case 8: hipLaunchKernelGGL((reduce_kernel<E, 8>), dim3(blocks_for(ReduceUnroll<8>::U)), blk, 0, s, a, total_bytes); break;
-    default: return hipErrorInvalidValue;
-    }
+template <class E, int N>
+hipError_t launch_reduce_n(const RowArgs &a, int64_t row_bytes, int64_t first_row, int64_t row_step, int64_t rows,
+                           hipStream_t s) {
+    constexpr int64_t span = 256 * ReduceUnroll<N>::U * 16;
+    ReduceSpan sp{row_bytes, first_row, row_step, (row_bytes + span - 1) / span};
+    const int64_t blocks = rows * sp.spans_per_row;
+    if (blocks <= 0) return hipSuccess;
+    if (blocks > 0x7fffffff) return hipErrorInvalidValue; // grid dimension limit
+    hipLaunchKernelGGL((reduce_kernel<E, N>), dim3((unsigned)blocks), dim3(256), 0, s, a, sp);
     return hipGetLastError();
+}
+
+// Stage A over rows first_row, first_row + row_step, ... (`rows` of them), each row_bytes long.
+template <class E>
+hipError_t launch_reduce_e(int n, const RowArgs &a, int64_t row_bytes, int64_t first_row, int64_t row_step, int64_t rows,
+                           hipStream_t s) {
+    switch (n) {
+    case 2: return launch_reduce_n<E, 2>(a, row_bytes, first_row, row_step, rows, s);
+    case 4: return launch_reduce_n<E, 4>(a, row_bytes, first_row, row_step, rows, s);
+    case 8: return launch_reduce_n<E, 8>(a, row_bytes, first_row, row_step, rows, s);
+    }
+    return hipErrorInvalidValue;
 }
 
 } // namespace tde

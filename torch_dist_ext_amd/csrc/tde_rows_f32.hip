@@ -7,8 +7,9 @@ hipError_t launch_rows_f32(int n, int vpt, int q, bool wn, const RowArgs &a, con
     return launch_rows_e<ElemF32>(n, vpt, q, wn, a, g, s);
 }
 
-hipError_t launch_reduce_f32(int n, const RowArgs &a, int64_t total_vecs, hipStream_t s) {
-    return launch_reduce_e<ElemF32>(n, a, total_vecs, s);
+hipError_t launch_reduce_f32(int n, const RowArgs &a, int64_t row_bytes, int64_t first_row, int64_t row_step, int64_t rows,
+                             hipStream_t s) {
+    return launch_reduce_e<ElemF32>(n, a, row_bytes, first_row, row_step, rows, s);
 }
 
 } // namespace tde
