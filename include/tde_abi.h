@@ -141,6 +141,17 @@ int tde_plan(const tde_problem *problem, tde_plan_out *plan);
    (impl.h:500-535) for the arithmetic of one rank; quant outputs extend it. */
 int tde_reduce_rms(const tde_problem *problem, const tde_buffers *buffers, void *hip_stream);
 
+/* The two launches of the staged algorithms (problem->algo must be TDE_ALGO_STAGED or TDE_ALGO_STAGED_OWNED,
+   else TDE_EALGO), one at a time, for a caller that puts its own exchange between them as the reference's
+   two-shot kernel does with its barrier (impl.h:377-380):
+   tde_stage_reduce = the reduce-scatter body (impl.h:365-377): sums the partials of all rows, or of rows ==
+   rank (mod nranks), into buffers->stage; only partial[], partial_table and stage are read from `buffers`.
+   tde_stage_norm = the body after the barrier (impl.h:381-393): residual add + norm (+quant) of every row of
+   buffers->stage; partial[] and partial_table are ignored.
+   tde_reduce_rms with the same problem is exactly tde_stage_reduce followed by tde_stage_norm. */
+int tde_stage_reduce(const tde_problem *problem, const tde_buffers *buffers, void *hip_stream);
+int tde_stage_norm(const tde_problem *problem, const tde_buffers *buffers, void *hip_stream);
+
 /* Tuning hook for sweeps and tests: force vectors-per-thread (1,2,4), rows per workgroup and a cap
    on the grid (rows beyond it are covered by a grid-stride loop).  0 restores the automatic choice
    for that field.  Process-wide, not thread-safe.  No counterpart in the reference, whose

@@ -34,10 +34,12 @@ def bits_equal(a: torch.Tensor, b: torch.Tensor) -> bool:
 
 
 def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, write_norm=None, use_table=False,
-            rank=0, device="cuda:0", static_scale=0.0, stage_init=None):
+            rank=0, device="cuda:0", static_scale=0.0, stage_init=None, calls=None):
     """Run the HIP path through the C ABI (tde_reduce_rms) on CPU inputs; returns CPU outputs.
     parts: [N,T,H] tensor or list of N [T,H] tensors.  stage_init: [T,H] initial content of the stage
-    buffer (staged algorithms); the stage is then returned as out["stage"]."""
+    buffer (staged algorithms); the stage is then returned as out["stage"].  calls: sequence of
+    (phases, rank) issued in order on the same buffers instead of the one tde_reduce_rms call, e.g.
+    [(("reduce",), 0), (("reduce",), 1), (("norm",), 0)]."""
     dev = torch.device(device)
     n = len(parts)
     T, H = residual.shape
@@ -62,8 +64,6 @@ def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, wri
         d_stage = stage_init.contiguous().to(dev)
     elif algo in (_capi.ALGO_STAGED, _capi.ALGO_STAGED_OWNED):
         d_stage = torch.empty_like(d_res)
-    prob = _capi.make_problem(DTYPE_CODE[dtype], n, T, H, eps, quant=qm, algo=algo, write_norm=int(bool(write_norm)),
-                              rank=rank, static_scale=static_scale)
     ptrs = [p.data_ptr() for p in d_parts]
     table = None
     d_table = None
@@ -72,12 +72,15 @@ def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, wri
         table = d_table.data_ptr()
         ptrs = [p if r == rank else None for r, p in enumerate(ptrs)]
     stream = torch.cuda.current_stream(dev).cuda_stream
-    _capi.reduce_rms(prob, ptrs, d_res.data_ptr(), d_res_out.data_ptr(), d_gamma.data_ptr(),
-                     norm_out=d_norm.data_ptr() if d_norm is not None else None,
-                     q_out=d_q.data_ptr() if d_q is not None else None,
-                     scale_out=d_scale.data_ptr() if d_scale is not None else None,
-                     stage=d_stage.data_ptr() if d_stage is not None else None,
-                     partial_table=table, stream=stream)
+    for phases, call_rank in (calls or [(("reduce", "norm"), rank)]):
+        prob = _capi.make_problem(DTYPE_CODE[dtype], n, T, H, eps, quant=qm, algo=algo, write_norm=int(bool(write_norm)),
+                                  rank=call_rank, static_scale=static_scale)
+        _capi.reduce_rms(prob, ptrs, d_res.data_ptr(), d_res_out.data_ptr(), d_gamma.data_ptr(),
+                         norm_out=d_norm.data_ptr() if d_norm is not None else None,
+                         q_out=d_q.data_ptr() if d_q is not None else None,
+                         scale_out=d_scale.data_ptr() if d_scale is not None else None,
+                         stage=d_stage.data_ptr() if d_stage is not None else None,
+                         partial_table=table, stream=stream, phases=phases)
     torch.cuda.synchronize(dev)
     out = {"residual_out": d_res_out.cpu()}
     if stage_init is not None:

@@ -106,6 +106,36 @@ def test_staged_owned_rows(cuda_device, n, rank, tokens, hidden, dtype, quant):
         assert torch.isnan(c["residual_out"][~own].float()).all()
 
 
+@pytest.mark.parametrize("n,tokens,hidden,dtype,quant", [
+    (4, 130, 2048, torch.bfloat16, "fp8_token"), (8, 67, 4096, torch.float16, "fp8_group"),
+    (2, 129, 1024, torch.float32, "none"), (8, 5, 8192, torch.bfloat16, "int8_token"),
+])
+def test_two_shot_emulated_by_phase_calls(cuda_device, n, tokens, hidden, dtype, quant):
+    """The whole two-shot on one GPU: N tde_stage_reduce calls, one per rank's share of the rows, all
+    into the same (NaN-filled) stage, then one tde_stage_norm.  Bit-identical to the fused path."""
+    p, r, g = eager.make_inputs(n, tokens, hidden, dtype, 1.0, seed=400 + n)
+    a = run_hip(p, r, g, 1e-6, quant, algo=_capi.ALGO_FUSED)
+    calls = [(("reduce",), k) for k in range(n)] + [(("norm",), 0)]
+    b = run_hip(p, r, g, 1e-6, quant, algo=_capi.ALGO_STAGED_OWNED, calls=calls,
+                stage_init=torch.full((tokens, hidden), float("nan"), dtype=dtype))
+    assert bits_equal(b.pop("stage"), _rank_order_sum(p))
+    for k in a:
+        assert bits_equal(a[k], b[k]), k
+    # and the all-rows staged algorithm split the same way
+    c = run_hip(p, r, g, 1e-6, quant, algo=_capi.ALGO_STAGED, calls=[(("reduce",), 0), (("norm",), 0)])
+    for k in a:
+        assert bits_equal(a[k], c[k]), k
+
+
+def test_phase_calls_need_a_staged_algorithm(cuda_device):
+    p, r, g = eager.make_inputs(4, 8, 1024, torch.bfloat16, 1.0, seed=5)
+    for phases in (("reduce",), ("norm",)):
+        with pytest.raises(_capi.TdeError) as ei:
+            run_hip(p, r, g, 1e-6, "none", algo=_capi.ALGO_FUSED, calls=[(phases, 0)],
+                    stage_init=torch.zeros(8, 1024, dtype=torch.bfloat16))
+        assert ei.value.status == _capi.EALGO
+
+
 def test_pointer_table_equals_direct(cuda_device):
     p, r, g = eager.make_inputs(8, 33, 4096, torch.bfloat16, 0.5, seed=22)
     a = run_hip(p, r, g, 1e-5, "fp8_token")

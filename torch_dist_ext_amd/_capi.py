@@ -17,7 +17,8 @@ ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, ALGO_STAGED_OWNED = 0, 1, 2, 3
 
 # Every symbol include/tde_abi.h declares.
 EXPORTS = (
-    "tde_abi_version", "tde_status_string", "tde_last_hip_error", "tde_plan", "tde_reduce_rms", "tde_tune_override", "tde_probe_copy",
+    "tde_abi_version", "tde_status_string", "tde_last_hip_error", "tde_plan", "tde_reduce_rms", "tde_stage_reduce", "tde_stage_norm",
+    "tde_tune_override", "tde_probe_copy",
     "tde_workspace_create", "tde_workspace_destroy", "tde_workspace_slot", "tde_workspace_stage",
     "tde_workspace_slot_bytes", "tde_workspace_nranks", "tde_workspace_fill_table",
 )
@@ -73,6 +74,9 @@ def load():
     lib.tde_plan.argtypes = [ctypes.POINTER(Problem), ctypes.POINTER(PlanOut)]
     lib.tde_reduce_rms.restype = ctypes.c_int
     lib.tde_reduce_rms.argtypes = [ctypes.POINTER(Problem), ctypes.POINTER(Buffers), ctypes.c_void_p]
+    for fn in (lib.tde_stage_reduce, lib.tde_stage_norm):
+        fn.restype = ctypes.c_int
+        fn.argtypes = [ctypes.POINTER(Problem), ctypes.POINTER(Buffers), ctypes.c_void_p]
     lib.tde_tune_override.restype = ctypes.c_int
     lib.tde_tune_override.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
     lib.tde_probe_copy.restype = ctypes.c_int
@@ -121,16 +125,20 @@ def plan(problem):
 
 
 def reduce_rms(problem, partials, residual_in, residual_out, gamma, norm_out=None, q_out=None, scale_out=None,
-               stage=None, partial_table=None, stream=None):
+               stage=None, partial_table=None, stream=None, phases=("reduce", "norm")):
     """tde_reduce_rms with raw device addresses (ints).  `partials` is a sequence of addresses (None
-    entries are taken from partial_table).  Raises TdeError on a non-zero status."""
+    entries are taken from partial_table).  phases=("reduce",) / ("norm",) calls tde_stage_reduce /
+    tde_stage_norm instead.  Raises TdeError on a non-zero status."""
     b = Buffers()
     for r, p in enumerate(partials):
         b.partial[r] = p
     b.partial_table = partial_table
     b.residual_in, b.residual_out, b.norm_out, b.gamma = residual_in, residual_out, norm_out, gamma
     b.q_out, b.scale_out, b.stage = q_out, scale_out, stage
-    check(load().tde_reduce_rms(ctypes.byref(problem), ctypes.byref(b), stream))
+    lib = load()
+    fn = {("reduce", "norm"): lib.tde_reduce_rms, ("reduce",): lib.tde_stage_reduce,
+          ("norm",): lib.tde_stage_norm}[tuple(phases)]
+    check(fn(ctypes.byref(problem), ctypes.byref(b), stream))
 
 
 def tune_override(vecs_per_thread=0, rows_per_block=0, max_grid=0):

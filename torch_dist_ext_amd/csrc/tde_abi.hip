@@ -186,7 +186,10 @@ int tde_plan(const tde_problem *problem, tde_plan_out *plan) {
     return TDE_OK;
 }
 
-int tde_reduce_rms(const tde_problem *p, const tde_buffers *b, void *hip_stream) {
+namespace {
+enum : int { kPhaseReduce = 1, kPhaseNorm = 2 };
+
+int run_phases(const tde_problem *p, const tde_buffers *b, void *hip_stream, int phases) {
     tde::Geometry g{};
     const int st = validate(p, &g);
     if (st != TDE_OK) return st;
@@ -195,15 +198,20 @@ int tde_reduce_rms(const tde_problem *p, const tde_buffers *b, void *hip_stream)
     const bool quant = p->quant != TDE_QUANT_NONE;
     const bool wn = !quant || p->write_norm != 0;
     const bool staged = p->algo == TDE_ALGO_STAGED || p->algo == TDE_ALGO_STAGED_OWNED;
+    const bool both = phases == (kPhaseReduce | kPhaseNorm);
+    if (!both && !staged) return TDE_EALGO; // a single phase exists only in the staged algorithms
+    const bool reads_partials = !staged || (phases & kPhaseReduce);
 
-    for (int r = 0; r < p->nranks; ++r) {
+    for (int r = 0; reads_partials && r < p->nranks; ++r) {
         if (b->partial[r] == nullptr && b->partial_table == nullptr) return TDE_EINVAL;
         if (!aligned16(b->partial[r])) return TDE_EALIGN;
     }
-    if (!b->residual_in || !b->residual_out || !b->gamma) return TDE_EINVAL;
-    if (wn && !b->norm_out) return TDE_EINVAL;
-    if (quant && !b->q_out) return TDE_EINVAL;
-    if (quant && p->quant != TDE_QUANT_FP8_STATIC && !b->scale_out) return TDE_EINVAL;
+    if (phases & kPhaseNorm) {
+        if (!b->residual_in || !b->residual_out || !b->gamma) return TDE_EINVAL;
+        if (wn && !b->norm_out) return TDE_EINVAL;
+        if (quant && !b->q_out) return TDE_EINVAL;
+        if (quant && p->quant != TDE_QUANT_FP8_STATIC && !b->scale_out) return TDE_EINVAL;
+    }
     if (staged && !b->stage) return TDE_EALGO;
     if (!aligned16(b->residual_in) || !aligned16(b->residual_out) || !aligned16(b->gamma) ||
         !aligned16(b->norm_out) || !aligned16(b->stage) || !aligned16(b->partial_table))
@@ -233,7 +241,7 @@ int tde_reduce_rms(const tde_problem *p, const tde_buffers *b, void *hip_stream)
 
     int n = p->nranks;
     hipError_t e = hipSuccess;
-    if (staged) {
+    if (staged && (phases & kPhaseReduce)) {
         // All rows as one span of bytes, or only this rank's share (rows == rank mod nranks) row by row.
         const int64_t row_bytes = (int64_t)g.nvec * 16;
         int64_t span_bytes = p->tokens * row_bytes, first = 0, step = 1, rows = 1;
@@ -249,6 +257,9 @@ int tde_reduce_rms(const tde_problem *p, const tde_buffers *b, void *hip_stream)
         case TDE_F32: e = tde::launch_reduce_f32(n, a, span_bytes, first, step, rows, stream); break;
         }
         if (e != hipSuccess) return hip_fail(e);
+    }
+    if (!(phases & kPhaseNorm)) return TDE_OK;
+    if (staged) {
         for (int r = 0; r < tde::kMaxKernelRanks; ++r) a.part[r] = nullptr;
         a.part[0] = b->stage;
         a.table = nullptr;
@@ -261,6 +272,19 @@ int tde_reduce_rms(const tde_problem *p, const tde_buffers *b, void *hip_stream)
     }
     if (e != hipSuccess) return hip_fail(e);
     return TDE_OK;
+}
+} // namespace
+
+int tde_reduce_rms(const tde_problem *p, const tde_buffers *b, void *hip_stream) {
+    return run_phases(p, b, hip_stream, kPhaseReduce | kPhaseNorm);
+}
+
+int tde_stage_reduce(const tde_problem *p, const tde_buffers *b, void *hip_stream) {
+    return run_phases(p, b, hip_stream, kPhaseReduce);
+}
+
+int tde_stage_norm(const tde_problem *p, const tde_buffers *b, void *hip_stream) {
+    return run_phases(p, b, hip_stream, kPhaseNorm);
 }
 
 // ---- emulated peer workspace ----------------------------------------------------------------
