@@ -262,6 +262,10 @@ __global__ void __launch_bounds__(1024 / VPT)
     __attribute__((amdgpu_waves_per_eu(VPT == 1 ? 8 : (VPT == 2 ? 5 : 3)))) row_kernel(const RowArgs a) {
     constexpr int VEC = E::VEC;
     constexpr int NP = (N == 0) ? 1 : N;
+    // Where residual_out is stored.  With 8 partials per row the stores go out together with the row's other
+    // output at the end (one write burst per row: 0.9 % faster on 8 x [2048, 8192] bf16 -> fp8); with fewer
+    // partials storing as soon as the sum is known measures 0.6-1.3 % faster.
+    constexpr bool LATE_RESIDUAL = (N >= 8);
     __shared__ float lds_sum[2][kMaxWavesPerBlock];
     __shared__ float lds_max[2][kMaxWavesPerBlock];
 
@@ -353,7 +357,7 @@ __global__ void __launch_bounds__(1024 / VPT)
 #pragma unroll
             for (int i = 0; i < VEC; ++i) x[i] = s[i] + res[i];
             xraw[j] = E::pack(x);
-            rsrc_store16(res_out, lane_off[j], xraw[j]);
+            if constexpr (!LATE_RESIDUAL) rsrc_store16(res_out, lane_off[j], xraw[j]);
             E::unpack(xraw[j], x);
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
@@ -405,6 +409,11 @@ __global__ void __launch_bounds__(1024 / VPT)
             }
         }
 
+        if constexpr (LATE_RESIDUAL && Q == TDE_QUANT_NONE) {
+#pragma unroll
+            for (int j = 0; j < VPT; ++j) rsrc_store16(res_out, lane_off[j], xraw[j]);
+        }
+
         // ---- dynamic quant epilogue ---------------------------------------------------------------
         if constexpr (Q != TDE_QUANT_NONE) {
             constexpr float QMAX = (Q == TDE_QUANT_INT8_TOKEN) ? 127.0f : 448.0f;
@@ -436,6 +445,10 @@ __global__ void __launch_bounds__(1024 / VPT)
                 if (row_ok && t == 0) ((TDE_GLOBAL float *)a.scale_out)[row] = sc;
             }
             const rsrc_t q_out = row_rsrc(a.q_out, row * (int64_t)a.hidden, row_ok ? (uint32_t)a.hidden : 0u);
+            if constexpr (LATE_RESIDUAL) {
+#pragma unroll
+                for (int j = 0; j < VPT; ++j) rsrc_store16(res_out, lane_off[j], xraw[j]);
+            }
 #pragma unroll
             for (int j = 0; j < VPT; ++j) {
                 float y[VEC], q[VEC];
