@@ -53,7 +53,8 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     const int vec = 16 / eb;
     const int64_t nvec = p->hidden / vec;
     if (nvec > kMaxBlock) return TDE_EHIDDEN; // as the reference: one 16-byte vector per thread, 1024 threads
-    if (p->tokens > 0 && p->tokens * p->hidden / p->hidden != p->tokens) return TDE_ESHAPE;
+    int64_t total_bytes = 0; // tokens * hidden * elem must be addressable with 64-bit signed offsets
+    if (__builtin_mul_overflow(p->tokens, p->hidden * eb, &total_bytes)) return TDE_ESHAPE;
 
     // Vectors per thread.  Four vectors per thread (small workgroups, many loads in flight per thread,
     // few wavefronts to synchronize per row) win where they fill their lanes: rows of 896+ vectors, and
