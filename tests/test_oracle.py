@@ -3,6 +3,8 @@ order-sensitivity vector, integer-arithmetic conversions against torch's, the re
 CPU check (restated, and the reference-built copy where oracle/_ref exists), and — for the quant
 definitions, which the reference does not have — textbook encoders and dequantization properties."""
 import math
+import os
+import sys
 
 import numpy as np
 import pytest
@@ -289,3 +291,22 @@ def test_golden_fixtures_reproduce():
         if quant != "none":
             assert np.array_equal(out["q"].view(torch.uint8).numpy(), z[name + "/q"]), name
             assert np.array_equal(out["scale"].numpy(), z[name + "/scale"]), name
+
+
+@pytest.mark.parametrize("key", ["c2", "c3", "c4", "c5@4096"])
+def test_full_size_digests_reproduce(key):
+    """tests/golden/digests.json (written by tests/golden/make_digests.py): the oracle regenerates the
+    same residual_out bits from the seeds; the outputs that follow torch's mean() are compared only on
+    a host with the vector ISA the digests were made on."""
+    import json
+    sys.path.insert(0, os.path.join(os.path.dirname(__file__), "golden"))
+    import make_digests
+    with open(os.path.join(os.path.dirname(__file__), "golden", "digests.json")) as f:
+        want = json.load(f)
+    name, _, tok = key.partition("@")
+    got = make_digests.digest_case(name, int(tok) if tok else None)
+    if got["inputs"] != want[key]["inputs"]:
+        pytest.skip("this host's torch generates different inputs from the same seeds")
+    assert got["residual_out"] == want[key]["residual_out"]
+    if torch.backends.cpu.get_cpu_capability() == want["cpu_capability"]:
+        assert got == want[key]

@@ -1,6 +1,8 @@
 """GPU parity: the HIP path, called through the C ABI (tde_reduce_rms), against the CPU oracle on the
 same seeded inputs.  Bar: residual bit-exact, normed <= 1 ulp, codes <= 1 quant step, scales <= 1e-6
 relative (test/test_all_reduce_fusion.py:23-28,75-76 is the composition the oracle restates)."""
+import os
+
 import pytest
 import torch
 
@@ -472,3 +474,26 @@ def test_quant_with_scales_outside_the_fast_division_range(cuda_device, dtype, q
     p, r, g = eager.make_inputs(4, 11, 1024, torch.float32, 1.0, seed=71)
     p, r, g = p.to(dtype), r.to(dtype), (g * gscale).to(dtype)
     _case("tiny-scale", p, r, g, 1e-6, quant)
+
+
+@pytest.mark.parametrize("key", ["c2", "c3", "c4", "c5@4096"])
+def test_full_size_residual_matches_committed_digest(cuda_device, key):
+    """residual_out is bit-exact by contract: its SHA-256 at full size must equal the digest the CPU
+    oracle produced when tests/golden/digests.json was written (inputs regenerate from their seeds;
+    the case is skipped if this host's torch generates different inputs)."""
+    import hashlib
+    import json
+    with open(os.path.join(os.path.dirname(__file__), "golden", "digests.json")) as f:
+        want = json.load(f)[key]
+    name, _, tok = key.partition("@")
+    p, r, g, eps, quant = eager.make_config(name, tokens=int(tok) if tok else None)
+
+    def sha(*ts):
+        h = hashlib.sha256()
+        for t in ts:
+            h.update(t.contiguous().view(torch.uint8).numpy().tobytes())
+        return h.hexdigest()
+    if sha(p, r, g) != want["inputs"]:
+        pytest.skip("this host's torch generates different inputs from the same seeds")
+    out = run_hip(p, r, g, eps, quant)
+    assert sha(out["residual_out"]) == want["residual_out"]
