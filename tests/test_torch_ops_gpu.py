@@ -90,6 +90,13 @@ def test_error_paths_raise(tde, cuda_device):
         tde.peer_partial(1, torch.zeros((64, 256), dtype=torch.bfloat16, device=cuda_device))
     with pytest.raises(RuntimeError, match="rank"):
         tde.CommWorkspace(5, 4, 256, 4096)
+    # rows that do not fit the workspace slots (4096 bytes here) are refused, not read past the slot
+    big = torch.zeros((16, 256), dtype=torch.bfloat16, device=cuda_device)
+    with pytest.raises(RuntimeError, match="workspace slots hold 4096"):
+        tde.allreduce_rms_fusion_impl(0, 2, big, big, g, torch.empty_like(big), torch.empty_like(big), 1e-6, ws)
+    # so is a table that no live workspace handed out
+    with pytest.raises(RuntimeError, match="not a pointer table handed out"):
+        tde.allreduce_rms_fusion_impl(0, 2, x, x, g, torch.empty_like(x), torch.empty_like(x), 1e-6, ws.clone())
     y = torch.zeros((4, 8200), dtype=torch.bfloat16, device=cuda_device)
     with pytest.raises(AssertionError):
         tde.allreduce_rms(0, 2, y, y, torch.ones(8200, dtype=torch.bfloat16, device=cuda_device), 1e-6, ws)
@@ -136,3 +143,27 @@ def test_static_quant_op(tde, cuda_device):
                                                                tde.QUANT_FP8_STATIC, False, 0.01)
     torch.cuda.synchronize()
     assert s.numel() == 0 and no.numel() == 0 and bits_equal(q.cpu(), out["q"].cpu())
+
+
+def test_slot_alias_keeps_the_workspace_alive(tde, cuda_device):
+    """A tensor returned by peer_partial/stage aliases workspace memory and must keep it allocated after
+    the workspace object itself is dropped; a table whose workspace is gone is refused."""
+    import gc
+    ref = torch.zeros((8, 512), dtype=torch.bfloat16, device=cuda_device)
+    ws = tde.CommWorkspace(0, 2, 256, 8 * 512 * 2)
+    table = ws.get_workspace(ref)
+    alias = ws.peer_partial(1, ref)
+    del ws
+    gc.collect()
+    alias.fill_(3.0)
+    torch.cuda.synchronize()
+    assert float(alias.float().sum().item()) == 3.0 * 8 * 512
+    g = torch.ones((512,), dtype=torch.bfloat16, device=cuda_device)
+    # the alias still owns the workspace, so its table stays valid
+    out = torch.empty_like(ref)
+    tde.allreduce_rms_fusion_impl(0, 2, ref, ref, g, torch.empty_like(ref), out, 1e-6, table)
+    torch.cuda.synchronize()
+    del alias
+    gc.collect()
+    with pytest.raises(RuntimeError, match="not a pointer table handed out"):
+        tde.allreduce_rms_fusion_impl(0, 2, ref, ref, g, torch.empty_like(ref), out, 1e-6, table)

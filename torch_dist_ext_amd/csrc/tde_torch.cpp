@@ -13,7 +13,9 @@
 #include <unistd.h>
 
 #include <cstring>
+#include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "tde_abi.h"
@@ -43,6 +45,30 @@ int32_t dtype_code(const Tensor &t) {
     return -1;
 }
 
+// Pointer tables handed out by CommWorkspace::get_workspace, keyed by their device address, with the size of
+// the slots they point to.  The operators receive only the table tensor (the reference's signature), so this
+// is how they learn how many bytes of each slot exist: a call whose rows do not fit is refused instead of
+// reading past a slot.
+std::mutex g_tables_mutex;
+std::unordered_map<const void *, int64_t> g_table_slot_bytes;
+
+void register_table(const void *table, int64_t slot_bytes) {
+    const std::lock_guard<std::mutex> lock(g_tables_mutex);
+    g_table_slot_bytes[table] = slot_bytes;
+}
+
+void unregister_table(const void *table) {
+    const std::lock_guard<std::mutex> lock(g_tables_mutex);
+    g_table_slot_bytes.erase(table);
+}
+
+// -1 if `table` was not handed out by a live CommWorkspace.
+int64_t table_slot_bytes(const void *table) {
+    const std::lock_guard<std::mutex> lock(g_tables_mutex);
+    const auto it = g_table_slot_bytes.find(table);
+    return it == g_table_slot_bytes.end() ? -1 : it->second;
+}
+
 void check_row_tensor(const Tensor &t, const Tensor &like, const char *name) {
     TORCH_CHECK(t.is_cuda(), name, " must be a GPU tensor");
     TORCH_CHECK(t.device() == like.device(), name, " is on a different device than allreduce_in");
@@ -64,7 +90,10 @@ public:
         check_status(tde_workspace_create((int32_t)world_size, size_in_bytes, &ws_), "CommWorkspace");
     }
 
-    ~CommWorkspace() override { tde_workspace_destroy(ws_); }
+    ~CommWorkspace() override {
+        if (table_.defined()) unregister_table(table_.data_ptr());
+        tde_workspace_destroy(ws_);
+    }
 
     // The reference returns the IPC handle of its allocation.  Nothing is exported here: the 64
     // bytes carry a tag, the process id, the rank and the address of slot `rank`.
@@ -105,7 +134,9 @@ public:
         auto host = at::empty({entries * (int64_t)sizeof(void *)}, at::TensorOptions().dtype(at::kByte).device(at::kCPU));
         check_status(tde_workspace_fill_table(ws_, reinterpret_cast<void **>(host.data_ptr()), (int32_t)entries),
                      "get_workspace");
+        if (table_.defined()) unregister_table(table_.data_ptr());
         table_ = host.to(ref.device());
+        register_table(table_.data_ptr(), size_in_bytes_);
         return table_;
     }
 
@@ -117,7 +148,7 @@ public:
         const int64_t bytes = ref.numel() * (int64_t)ref.element_size();
         TORCH_CHECK(bytes <= size_in_bytes_, "peer_partial: ", bytes, " bytes exceed the slot size ", size_in_bytes_);
         TORCH_CHECK(ref.is_cuda() && ref.device().index() == device_, "peer_partial: ref must live on the workspace's GPU");
-        return at::from_blob(tde_workspace_slot(ws_, (int32_t)r), ref.sizes(), ref.options());
+        return alias(tde_workspace_slot(ws_, (int32_t)r), ref);
     }
 
     void set_peer_partial(int64_t r, const Tensor &src) {
@@ -129,7 +160,7 @@ public:
     Tensor stage(const Tensor &ref) {
         const int64_t bytes = ref.numel() * (int64_t)ref.element_size();
         TORCH_CHECK(bytes <= size_in_bytes_, "stage: ", bytes, " bytes exceed the slot size ", size_in_bytes_);
-        return at::from_blob(tde_workspace_stage(ws_, (int32_t)rank_), ref.sizes(), ref.options());
+        return alias(tde_workspace_stage(ws_, (int32_t)rank_), ref);
     }
 
     int64_t rank() const { return rank_; }
@@ -137,6 +168,13 @@ public:
     int64_t size_in_bytes() const { return size_in_bytes_; }
 
 private:
+    // A tensor like `ref` over workspace memory.  It holds a reference to this object, so the memory
+    // outlives every such tensor.
+    Tensor alias(void *ptr, const Tensor &ref) {
+        auto self = c10::intrusive_ptr<CommWorkspace>::unsafe_reclaim_from_nonowning(this);
+        return at::from_blob(ptr, ref.sizes(), [self](void *) {}, ref.options());
+    }
+
     int64_t rank_, world_size_, nblocks_, size_in_bytes_;
     int device_ = 0;
     bool opened_ = false;
@@ -208,6 +246,23 @@ void run(Call &c, const Tensor &on) {
     check_status(tde_reduce_rms(&c.p, &c.b, stream), "torch_dist_ext");
 }
 
+// Points the call at the workspace's slots, with the caller's own partial read straight from allreduce_in.
+void use_table(Call &c, int64_t rank, int64_t nranks, const Tensor &allreduce_in, const Tensor &workspace) {
+    TORCH_CHECK(nranks == 2 || nranks == 4 || nranks == 8, "torch_dist_ext: ", tde_status_string(TDE_ENRANKS));
+    TORCH_CHECK(workspace.is_cuda() && workspace.scalar_type() == at::kByte && workspace.is_contiguous() &&
+                    workspace.numel() >= (3 * nranks + 5) * (int64_t)sizeof(void *),
+                "workspace must be the uint8 GPU pointer table returned by get_workspace for this world size");
+    TORCH_CHECK(rank >= 0 && rank < nranks && nranks <= TDE_MAX_RANKS, "rank/nranks out of range");
+    const int64_t slot_bytes = table_slot_bytes(workspace.data_ptr());
+    TORCH_CHECK(slot_bytes >= 0, "workspace is not a pointer table handed out by a live CommWorkspace's get_workspace "
+                                 "(pass that tensor itself, not a copy)");
+    const int64_t bytes = allreduce_in.numel() * (int64_t)allreduce_in.element_size();
+    TORCH_CHECK(bytes <= slot_bytes, "allreduce_in has ", bytes, " bytes but the workspace slots hold ", slot_bytes,
+                "; create the workspace (setup_env) with a larger size");
+    c.b.partial_table = reinterpret_cast<const void *const *>(workspace.data_ptr());
+    c.b.partial[rank] = allreduce_in.data_ptr();
+}
+
 // Reference entry point, verbatim signature (src/ops/all_reduce_fusion.h:42-43).  `workspace` is
 // the device pointer table from CommWorkspace::get_workspace; its first nranks entries are the
 // slots.  The caller's own partial is read straight from allreduce_in (the reference first copies
@@ -217,12 +272,7 @@ void allreduce_rms_fusion(int64_t rank, int64_t nranks, Tensor &allreduce_in, Te
     Call c;
     fill_common(c, rank, nranks, allreduce_in, residual_in, rms_gamma, residual_out, eps);
     fill_quant(c, TDE_QUANT_NONE, allreduce_in, norm_out, c10::nullopt, c10::nullopt);
-    TORCH_CHECK(workspace.is_cuda() && workspace.scalar_type() == at::kByte && workspace.is_contiguous() &&
-                    workspace.numel() >= (3 * nranks + 5) * (int64_t)sizeof(void *),
-                "workspace must be the uint8 GPU pointer table returned by get_workspace for this world size");
-    TORCH_CHECK(rank >= 0 && rank < nranks && nranks <= TDE_MAX_RANKS, "rank/nranks out of range");
-    c.b.partial_table = reinterpret_cast<const void *const *>(workspace.data_ptr());
-    c.b.partial[rank] = allreduce_in.data_ptr();
+    use_table(c, rank, nranks, allreduce_in, workspace);
     run(c, allreduce_in);
 }
 
@@ -234,12 +284,7 @@ void allreduce_rms_quant_fusion(int64_t rank, int64_t nranks, Tensor &allreduce_
     Call c;
     fill_common(c, rank, nranks, allreduce_in, residual_in, rms_gamma, residual_out, eps);
     fill_quant(c, quant_mode, allreduce_in, norm_out, q_out, scale_out, static_scale);
-    TORCH_CHECK(workspace.is_cuda() && workspace.scalar_type() == at::kByte && workspace.is_contiguous() &&
-                    workspace.numel() >= (3 * nranks + 5) * (int64_t)sizeof(void *),
-                "workspace must be the uint8 GPU pointer table returned by get_workspace for this world size");
-    TORCH_CHECK(rank >= 0 && rank < nranks && nranks <= TDE_MAX_RANKS, "rank/nranks out of range");
-    c.b.partial_table = reinterpret_cast<const void *const *>(workspace.data_ptr());
-    c.b.partial[rank] = allreduce_in.data_ptr();
+    use_table(c, rank, nranks, allreduce_in, workspace);
     run(c, allreduce_in);
 }
 
