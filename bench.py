@@ -191,14 +191,14 @@ def main():
                    else "achieved HBM GB/s, one rank's %d-partial reduce+residual+RMSNorm stage, quant=%s" % (N, quant)),
         "value": gbs_job, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": dt, "data": "synthetic",
+        "dtype": "f32", "data": "synthetic",   # arithmetic is fp32 throughout; storage types are in config
         "tokens_per_s": T / (wall / args.steps),
         "pct_of_hbm_peak": 100.0 * gbs_job / HBM_PEAK_GBS,
         "config": {"workload": "%s: N=%d partials [%d,%d] %s, residual add + RMSNorm + %s%s" % (
                        args.config, N, T, H, dt, quant,
                        {"staged": " (two launches through a stage buffer)",
                         "staged_owned": " (two launches; stage A over this rank's T/N rows only)"}.get(args.algo, "")),
-                   "algo": args.algo, "input_sets": nsets, "block_threads": plan.block_threads,
+                   "storage_dtype": dt, "output": quant, "algo": args.algo, "input_sets": nsets, "block_threads": plan.block_threads,
                    "grid_blocks": plan.grid_blocks, "algorithmic_bytes": bytes_per_launch},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None if staged else TRAFFIC_BYTES.get(args.config),
