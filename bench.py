@@ -204,6 +204,13 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None if staged else TRAFFIC_BYTES.get(args.config),
                      "kernel_avg_us": avg_ms * 1e3},
     }
+    info = _capi.device_info()
+    out["device"] = {"name": torch.cuda.get_device_properties(dev).name, "compute_units": info.compute_units,
+                     "memory_clock_khz": info.memory_clock_khz, "memory_bus_bits": info.memory_bus_bits,
+                     "hbm_bytes": info.total_memory_bytes,
+                     # transfers per reported memory clock that the published 8 TB/s corresponds to
+                     "peak_transfers_per_clock": (HBM_PEAK_GBS * 1e9 * 8 / (info.memory_bus_bits * info.memory_clock_khz * 1e3)
+                                                  if info.memory_bus_bits and info.memory_clock_khz else None)}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, cfg)
     print(json.dumps(out))

@@ -163,6 +163,20 @@ int tde_tune_override(int32_t vecs_per_thread, int32_t rows_per_block, int32_t m
    measuring the device's practical streaming ceiling.  No counterpart in the reference. */
 int tde_probe_copy(void *dst, const void *src, int64_t bytes, void *hip_stream);
 
+/* Properties of the current device as the HIP runtime reports them, for printing next to measured rates:
+   compute units, memory clock (kHz), memory bus width (bits; 0 where the runtime reports none) and total
+   device memory.  The clock is the runtime's figure, not the per-pin data rate: MI355X reports 2 000 000 kHz
+   x 8192 bits for HBM3E rated 8 TB/s, i.e. 3.9 transfers per reported clock.  No counterpart in the
+   reference, which hard-codes its block counts (impl.h:481-489). */
+typedef struct tde_device_info_out {
+    int32_t compute_units;
+    int32_t memory_clock_khz;
+    int32_t memory_bus_bits;
+    int32_t reserved;
+    int64_t total_memory_bytes;
+} tde_device_info_out;
+int tde_device_info(tde_device_info_out *out);
+
 /* ---- emulated peer workspace ----------------------------------------------------------------
    One allocation per emulated rank plays the role of that rank's IPC-mapped comm buffer
    (CommWorkspace, src/ops/all_reduce_fusion.cpp:63-96).  Each slot is 2*slot_bytes large: the

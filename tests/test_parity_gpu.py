@@ -497,3 +497,10 @@ def test_full_size_residual_matches_committed_digest(cuda_device, key):
         pytest.skip("this host's torch generates different inputs from the same seeds")
     out = run_hip(p, r, g, eps, quant)
     assert sha(out["residual_out"]) == want["residual_out"]
+
+
+def test_device_info(cuda_device):
+    info = _capi.device_info()
+    assert info.compute_units == torch.cuda.get_device_properties(0).multi_processor_count
+    assert info.total_memory_bytes == torch.cuda.get_device_properties(0).total_memory
+    assert info.memory_clock_khz >= 0 and info.memory_bus_bits >= 0

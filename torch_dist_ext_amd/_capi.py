@@ -18,7 +18,7 @@ ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, ALGO_STAGED_OWNED = 0, 1, 2, 3
 # Every symbol include/tde_abi.h declares.
 EXPORTS = (
     "tde_abi_version", "tde_status_string", "tde_last_hip_error", "tde_plan", "tde_reduce_rms", "tde_stage_reduce", "tde_stage_norm",
-    "tde_tune_override", "tde_probe_copy",
+    "tde_tune_override", "tde_probe_copy", "tde_device_info",
     "tde_workspace_create", "tde_workspace_destroy", "tde_workspace_slot", "tde_workspace_stage",
     "tde_workspace_slot_bytes", "tde_workspace_nranks", "tde_workspace_fill_table",
 )
@@ -46,6 +46,13 @@ class PlanOut(ctypes.Structure):
         ("block_threads", ctypes.c_int32), ("vecs_per_thread", ctypes.c_int32), ("rows_per_block", ctypes.c_int32),
         ("grid_blocks", ctypes.c_int32), ("reserved", ctypes.c_int32), ("algorithmic_bytes", ctypes.c_int64),
         ("scale_elems", ctypes.c_int64),
+    ]
+
+
+class DeviceInfo(ctypes.Structure):
+    _fields_ = [
+        ("compute_units", ctypes.c_int32), ("memory_clock_khz", ctypes.c_int32), ("memory_bus_bits", ctypes.c_int32),
+        ("reserved", ctypes.c_int32), ("total_memory_bytes", ctypes.c_int64),
     ]
 
 
@@ -81,6 +88,8 @@ def load():
     lib.tde_tune_override.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
     lib.tde_probe_copy.restype = ctypes.c_int
     lib.tde_probe_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+    lib.tde_device_info.restype = ctypes.c_int
+    lib.tde_device_info.argtypes = [ctypes.POINTER(DeviceInfo)]
     lib.tde_workspace_create.restype = ctypes.c_int
     lib.tde_workspace_create.argtypes = [ctypes.c_int32, ctypes.c_int64, ctypes.POINTER(ctypes.c_void_p)]
     lib.tde_workspace_destroy.restype = ctypes.c_int
@@ -143,6 +152,13 @@ def reduce_rms(problem, partials, residual_in, residual_out, gamma, norm_out=Non
 
 def tune_override(vecs_per_thread=0, rows_per_block=0, max_grid=0):
     check(load().tde_tune_override(vecs_per_thread, rows_per_block, max_grid))
+
+
+def device_info():
+    """tde_device_info for the current device -> DeviceInfo."""
+    out = DeviceInfo()
+    check(load().tde_device_info(ctypes.byref(out)))
+    return out
 
 
 def probe_copy(dst, src, nbytes, stream=None):

@@ -174,6 +174,29 @@ int tde_probe_copy(void *dst, const void *src, int64_t bytes, void *hip_stream) 
     return e == hipSuccess ? TDE_OK : hip_fail(e);
 }
 
+int tde_device_info(tde_device_info_out *out) {
+    if (out == nullptr) return TDE_EINVAL;
+    std::memset(out, 0, sizeof(*out));
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e);
+    int cu = 0, khz = 0, bits = 0;
+    e = hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return hip_fail(e);
+    // Clock and width are optional: a runtime that does not report them leaves zeros.
+    if (hipDeviceGetAttribute(&khz, hipDeviceAttributeMemoryClockRate, dev) != hipSuccess) khz = 0;
+    if (hipDeviceGetAttribute(&bits, hipDeviceAttributeMemoryBusWidth, dev) != hipSuccess) bits = 0;
+    (void)hipGetLastError();
+    size_t free_b = 0, total_b = 0;
+    e = hipMemGetInfo(&free_b, &total_b);
+    if (e != hipSuccess) return hip_fail(e);
+    out->compute_units = cu;
+    out->memory_clock_khz = khz;
+    out->memory_bus_bits = bits;
+    out->total_memory_bytes = (int64_t)total_b;
+    return TDE_OK;
+}
+
 int tde_plan(const tde_problem *problem, tde_plan_out *plan) {
     if (plan == nullptr) return TDE_EINVAL;
     tde::Geometry g{};
