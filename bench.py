@@ -183,6 +183,26 @@ def main():
     wall = time.perf_counter() - t0
     avg_ms = ev0.elapsed_time(ev1) / args.steps
 
+    # The same launches with the arithmetic removed (tde_probe_rows): what the access pattern alone takes
+    # on this box, in this process, over the same buffers.  It overwrites the outputs, hence after the timed run.
+    floor_us = None
+    if not staged:
+        def launch_floor(i):
+            st = lib.tde_probe_rows(prob_ref, call_refs[i % nsets], hip_stream)
+            if st != 0:
+                _capi.check(st)
+        for i in range(args.warmup):
+            launch_floor(i)
+        torch.cuda.synchronize(dev)
+        ev2 = torch.cuda.Event(enable_timing=True)
+        ev3 = torch.cuda.Event(enable_timing=True)
+        ev2.record(stream)
+        for i in range(args.steps):
+            launch_floor(i)
+        ev3.record(stream)
+        torch.cuda.synchronize(dev)
+        floor_us = ev2.elapsed_time(ev3) * 1e3 / args.steps
+
     ms_per_step = wall * 1e3 / args.steps
     gbs_job = bytes_per_launch / (wall / args.steps) / 1e9
     achieved = bytes_per_launch / (avg_ms * 1e-3) / 1e9
@@ -202,7 +222,10 @@ def main():
                    "grid_blocks": plan.grid_blocks, "algorithmic_bytes": bytes_per_launch},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None if staged else TRAFFIC_BYTES.get(args.config),
-                     "kernel_avg_us": avg_ms * 1e3},
+                     "kernel_avg_us": avg_ms * 1e3,
+                     # the same launches without arithmetic (same bytes, same access pattern), and their share of the peak
+                     "traffic_only_us": floor_us,
+                     "traffic_only_frac": (bytes_per_launch / (floor_us * 1e-6) / 1e9 / HBM_PEAK_GBS) if floor_us else None},
     }
     info = _capi.device_info()
     out["device"] = {"name": torch.cuda.get_device_properties(dev).name, "compute_units": info.compute_units,

@@ -163,6 +163,13 @@ int tde_tune_override(int32_t vecs_per_thread, int32_t rows_per_block, int32_t m
    measuring the device's practical streaming ceiling.  No counterpart in the reference. */
 int tde_probe_copy(void *dst, const void *src, int64_t bytes, void *hip_stream);
 
+/* Measurement aid: the memory traffic of tde_reduce_rms for the same problem and buffers with the arithmetic
+   removed -- same workgroups, lane mapping, load order and cache policies, every input byte read and every
+   output byte (scales excepted) written once, contents meaningless.  OVERWRITES residual_out, norm_out and
+   q_out.  Fused algorithm only (TDE_EALGO for the staged ones).  Timing it next to tde_reduce_rms shows how
+   far the kernel is from what its access pattern alone achieves.  No counterpart in the reference. */
+int tde_probe_rows(const tde_problem *problem, const tde_buffers *buffers, void *hip_stream);
+
 /* Properties of the current device as the HIP runtime reports them, for printing next to measured rates:
    compute units, memory clock (kHz), memory bus width (bits; 0 where the runtime reports none) and total
    device memory.  The clock is the runtime's figure, not the per-pin data rate: MI355X reports 2 000 000 kHz

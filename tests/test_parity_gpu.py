@@ -504,3 +504,27 @@ def test_device_info(cuda_device):
     assert info.compute_units == torch.cuda.get_device_properties(0).multi_processor_count
     assert info.total_memory_bytes == torch.cuda.get_device_properties(0).total_memory
     assert info.memory_clock_khz >= 0 and info.memory_bus_bits >= 0
+
+
+@pytest.mark.parametrize("n,tokens,hidden,dtype,quant,write_norm", [
+    (8, 70, 4096, torch.bfloat16, "fp8_token", False), (4, 33, 1024, torch.float16, "none", True),
+    (2, 300, 8192, torch.bfloat16, "int8_token", True), (4, 19, 508, torch.float32, "fp8_token", False),
+])
+def test_traffic_skeleton_touches_every_byte_once(cuda_device, n, tokens, hidden, dtype, quant, write_norm):
+    """tde_probe_rows reads every input vector and writes every output vector: its outputs are the
+    exclusive-or of all N+1 input rows (16 bytes at a time), folded to 8 or 4 bytes for the code rows."""
+    p, r, g = eager.make_inputs(n, tokens, hidden, dtype, 1.0, seed=77)
+    out = run_hip(p, r, g, 1e-6, quant, write_norm=write_norm, calls=[(("traffic",), 0)])
+    words = lambda t: t.contiguous().view(torch.int32).reshape(tokens, -1, 4)
+    x = words(r).clone()
+    for k in range(n):
+        x ^= words(p[k])
+    assert torch.equal(words(out["residual_out"]), x)
+    if write_norm or quant == "none":
+        assert torch.equal(words(out["norm_out"]), x)
+    if quant != "none":
+        q = out["q"].contiguous().view(torch.uint8).view(torch.int32)
+        if dtype == torch.float32:
+            assert torch.equal(q.reshape(tokens, -1), x[..., 0] ^ x[..., 1] ^ x[..., 2] ^ x[..., 3])
+        else:
+            assert torch.equal(q.reshape(tokens, -1, 2), torch.stack([x[..., 0] ^ x[..., 2], x[..., 1] ^ x[..., 3]], dim=-1))

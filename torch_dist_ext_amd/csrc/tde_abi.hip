@@ -215,7 +215,7 @@ int tde_plan(const tde_problem *problem, tde_plan_out *plan) {
 }
 
 namespace {
-enum : int { kPhaseReduce = 1, kPhaseNorm = 2 };
+enum : int { kPhaseReduce = 1, kPhaseNorm = 2, kTrafficOnly = 4 };
 
 int run_phases(const tde_problem *p, const tde_buffers *b, void *hip_stream, int phases) {
     tde::Geometry g{};
@@ -226,6 +226,11 @@ int run_phases(const tde_problem *p, const tde_buffers *b, void *hip_stream, int
     const bool quant = p->quant != TDE_QUANT_NONE;
     const bool wn = !quant || p->write_norm != 0;
     const bool staged = p->algo == TDE_ALGO_STAGED || p->algo == TDE_ALGO_STAGED_OWNED;
+    const bool traffic = phases == kTrafficOnly;
+    if (traffic) {
+        if (staged) return TDE_EALGO; // the skeleton mirrors the fused kernel only
+        phases = kPhaseReduce | kPhaseNorm;
+    }
     const bool both = phases == (kPhaseReduce | kPhaseNorm);
     if (!both && !staged) return TDE_EALGO; // a single phase exists only in the staged algorithms
     const bool reads_partials = !staged || (phases & kPhaseReduce);
@@ -269,6 +274,11 @@ int run_phases(const tde_problem *p, const tde_buffers *b, void *hip_stream, int
 
     int n = p->nranks;
     hipError_t e = hipSuccess;
+    if (traffic) {
+        const int code_bytes = quant ? (elem_bytes(p->dtype) == 4 ? 4 : 8) : 0;
+        e = tde::launch_traffic(n, g.vpt, code_bytes, wn, a, g, (uint32_t)g.nvec * 16u, stream);
+        return e == hipSuccess ? TDE_OK : hip_fail(e);
+    }
     if (staged && (phases & kPhaseReduce)) {
         // All rows as one span of bytes, or only this rank's share (rows == rank mod nranks) row by row.
         const int64_t row_bytes = (int64_t)g.nvec * 16;
@@ -313,6 +323,10 @@ int tde_stage_reduce(const tde_problem *p, const tde_buffers *b, void *hip_strea
 
 int tde_stage_norm(const tde_problem *p, const tde_buffers *b, void *hip_stream) {
     return run_phases(p, b, hip_stream, kPhaseNorm);
+}
+
+int tde_probe_rows(const tde_problem *p, const tde_buffers *b, void *hip_stream) {
+    return run_phases(p, b, hip_stream, kTrafficOnly);
 }
 
 // ---- emulated peer workspace ----------------------------------------------------------------
