@@ -486,12 +486,9 @@ __global__ void __launch_bounds__(1024 / VPT)
 // Stage A of the staged algorithm: s = T(sum of partials) for every element, no row structure.
 // One workgroup of 256 threads reduces a contiguous span of 256*U vectors (U vectors per thread,
 // all N*U loads in flight before the first add) and exits; spans past the end are cut by the buffer
-// resource's size, so there is no loop and no tail branch.
-template <int N>
-struct ReduceUnroll {
-    static constexpr int U = (N >= 8) ? 2 : 4;
-};
-
+// resource's size, so there is no loop and no tail branch.  U = 4 is the faster choice over the whole
+// tensor (8 partials x 32 MiB: 50.5 us against 52.9 us with U = 2); for single 16 KiB rows it would
+// leave one workgroup per row, and U = 2 (two per row) measures slightly faster there.
 // Which bytes stage A covers: `row_bytes` long rows first_row, first_row + row_step, ...; each row is cut
 // into spans_per_row spans.  The whole tensor as one long "row" (first_row 0) is the all-rows form; the
 // reference's two-shot share of one rank is rows == rank (mod nranks) (impl.h:365-366).
@@ -502,10 +499,9 @@ struct ReduceSpan {
     int64_t spans_per_row;
 };
 
-template <class E, int N>
+template <class E, int N, int U>
 __global__ void __launch_bounds__(256) reduce_kernel(const RowArgs a, const ReduceSpan sp) {
     constexpr int VEC = E::VEC;
-    constexpr int U = ReduceUnroll<N>::U;
     constexpr uint32_t SPAN = 256u * U * 16u; // bytes per workgroup
     const void *part[N];
 #pragma unroll
@@ -613,16 +609,23 @@ hipError_t launch_rows_e(int n, int vpt, int q, bool wn, const RowArgs &a, const
     return hipErrorInvalidValue;
 }
 
-template <class E, int N>
-hipError_t launch_reduce_n(const RowArgs &a, int64_t row_bytes, int64_t first_row, int64_t row_step, int64_t rows,
-                           hipStream_t s) {
-    constexpr int64_t span = 256 * ReduceUnroll<N>::U * 16;
+template <class E, int N, int U>
+hipError_t launch_reduce_nu(const RowArgs &a, int64_t row_bytes, int64_t first_row, int64_t row_step, int64_t rows,
+                            hipStream_t s) {
+    constexpr int64_t span = 256 * U * 16;
     ReduceSpan sp{row_bytes, first_row, row_step, (row_bytes + span - 1) / span};
     const int64_t blocks = rows * sp.spans_per_row;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffff) return hipErrorInvalidValue; // grid dimension limit
-    hipLaunchKernelGGL((reduce_kernel<E, N>), dim3((unsigned)blocks), dim3(256), 0, s, a, sp);
+    hipLaunchKernelGGL((reduce_kernel<E, N, U>), dim3((unsigned)blocks), dim3(256), 0, s, a, sp);
     return hipGetLastError();
+}
+
+template <class E, int N>
+hipError_t launch_reduce_n(const RowArgs &a, int64_t row_bytes, int64_t first_row, int64_t row_step, int64_t rows,
+                           hipStream_t s) {
+    if (N >= 8 && row_bytes <= 256 * 4 * 16) return launch_reduce_nu<E, N, 2>(a, row_bytes, first_row, row_step, rows, s);
+    return launch_reduce_nu<E, N, 4>(a, row_bytes, first_row, row_step, rows, s);
 }
 
 // Stage A over rows first_row, first_row + row_step, ... (`rows` of them), each row_bytes long.
