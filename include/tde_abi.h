@@ -35,12 +35,13 @@ typedef enum tde_status {
     TDE_OK = 0,
     TDE_EINVAL = 1,     /* null pointer / malformed struct */
     TDE_ENRANKS = 2,    /* nranks not in {2,4,8}; reference: assert(false) impl.h:526-534 */
-    TDE_EDTYPE = 3,     /* dtype not supported */
+    TDE_EDTYPE = 3,     /* dtype not supported (tde_probe_rows: not for TDE_F64) */
     TDE_ESHAPE = 4,     /* hidden*elem not a multiple of 16 bytes, tokens<0, hidden<=0 (impl.h:479-480) */
     TDE_EHIDDEN = 5,    /* hidden larger than the row kernel supports (reference: pkg assert, __init__.py:69) */
     TDE_EALIGN = 6,     /* a buffer is not 16-byte aligned (vec_t alignment, impl.h:208) */
-    TDE_EQUANT = 7,     /* unknown quant mode, group mode with hidden % 128 != 0, or a static scale that is not > 0 */
-    TDE_EALGO = 8,      /* unknown algorithm, or staged algorithm without a stage buffer */
+    TDE_EQUANT = 7,     /* unknown quant mode, group mode with hidden % 128 != 0, a static scale that is not > 0,
+                           or any quant mode with TDE_F64 */
+    TDE_EALGO = 8,      /* unknown algorithm, staged algorithm without a stage buffer or with TDE_F64 */
     TDE_EHIP = 9,       /* HIP runtime error; see tde_last_hip_error() */
     TDE_ERANK = 10,     /* rank outside [0,nranks) */
     TDE_ENOMEM = 11     /* device allocation failed */
@@ -50,7 +51,10 @@ typedef enum tde_status {
 typedef enum tde_dtype {
     TDE_BF16 = 0, /* __bfloat16 in the reference dispatch, src/ops/all_reduce_fusion.cpp:19-22 */
     TDE_F16 = 1,  /* __half,                              src/ops/all_reduce_fusion.cpp:14-17 */
-    TDE_F32 = 2   /* float,                               src/ops/all_reduce_fusion.cpp:29-33 */
+    TDE_F32 = 2,  /* float,                               src/ops/all_reduce_fusion.cpp:29-33 */
+    TDE_F64 = 3   /* double, admitted by the same macro;  src/ops/all_reduce_fusion.cpp:29-33.  Summed and normed
+                     in double as the eager composition does for double tensors (mean of squares in fp32,
+                     test_all_reduce_fusion.py:25); TDE_QUANT_NONE and the fused algorithm only */
 } tde_dtype;
 
 typedef enum tde_quant {

@@ -37,9 +37,10 @@ def reduce_residual(parts: torch.Tensor, residual_in: torch.Tensor) -> torch.Ten
     vectorized path; only the last few elements of the flattened tensor (the scalar tail when T*H is
     not a multiple of its vector chunk) are added in a different, host-ISA-dependent order
     (tests/test_oracle.py::test_torch_sum_dim0_is_rank_order_except_flat_tail)."""
-    acc = torch.zeros(parts.shape[1:], dtype=torch.float32)
+    acc_type = torch.float64 if parts.dtype == torch.float64 else torch.float32   # doubles are summed as doubles
+    acc = torch.zeros(parts.shape[1:], dtype=acc_type)
     for r in range(parts.shape[0]):
-        acc = acc + parts[r].float()
+        acc = acc + parts[r].to(acc_type)
     return acc.to(parts.dtype) + residual_in
 
 
@@ -121,12 +122,13 @@ def make_inputs(N, T, H, dtype, sigma=1.0, seed=0, outlier_channels=0, outlier_s
     partials ~ N(0, sigma), residual ~ N(0,1), gamma ~ U(0.5,1.5); optional fixed seeded set of
     `outlier_channels` columns multiplied by outlier_scale in every partial before the cast."""
     g = torch.Generator().manual_seed(seed)
-    parts = torch.randn((N, T, H), generator=g, dtype=torch.float32) * sigma
+    wide = torch.float64 if dtype == torch.float64 else torch.float32   # doubles get all their mantissa bits
+    parts = torch.randn((N, T, H), generator=g, dtype=wide) * sigma
     if outlier_channels:
         cols = torch.randperm(H, generator=g)[:outlier_channels]
         parts[:, :, cols] *= outlier_scale
-    residual = torch.randn((T, H), generator=g, dtype=torch.float32)
-    gamma = torch.rand((H,), generator=g, dtype=torch.float32) + 0.5
+    residual = torch.randn((T, H), generator=g, dtype=wide)
+    gamma = torch.rand((H,), generator=g, dtype=wide) + 0.5
     return parts.to(dtype), residual.to(dtype), gamma.to(dtype)
 
 

@@ -47,6 +47,8 @@ def _plan(**kw):
     (dict(hidden=8190), _capi.ESHAPE),      # 8190*2 bytes is not a multiple of 16 (impl.h:480)
     (dict(hidden=0), _capi.ESHAPE), (dict(tokens=-1), _capi.ESHAPE),
     (dict(tokens=1 << 60), _capi.ESHAPE),   # tokens * hidden * 2 overflows 64-bit byte offsets
+    (dict(dtype=_capi.F64, hidden=2050), _capi.EHIDDEN), (dict(dtype=_capi.F64, hidden=1025), _capi.ESHAPE),
+    (dict(dtype=_capi.F64, quant=_capi.QUANT_FP8_TOKEN), _capi.EQUANT), (dict(dtype=_capi.F64, algo=_capi.ALGO_STAGED), _capi.EALGO),
     (dict(hidden=8200), _capi.EHIDDEN),     # beyond 1024 vectors per row (the reference asserts hidden <= 8192)
     (dict(dtype=_capi.F32, hidden=4100), _capi.EHIDDEN),
     (dict(quant=9), _capi.EQUANT), (dict(quant=_capi.QUANT_FP8_GROUP, hidden=1032), _capi.EQUANT),

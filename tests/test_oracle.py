@@ -310,3 +310,22 @@ def test_full_size_digests_reproduce(key):
     assert got["residual_out"] == want[key]["residual_out"]
     if torch.backends.cpu.get_cpu_capability() == want["cpu_capability"]:
         assert got == want[key]
+
+
+def test_doubles_are_summed_as_doubles():
+    """For double tensors the eager composition (test/test_all_reduce_fusion.py:75) sums in double: a term
+    below fp32 resolution survives, and the order is still rank order (2^53 + 1 ties to even)."""
+    parts = torch.tensor([[[1.0, 2.0 ** 53]], [[2.0 ** -30, 1.0]], [[0.0, -(2.0 ** 53)]], [[0.0, 1.0]]], dtype=torch.float64)
+    res = torch.zeros((1, 2), dtype=torch.float64)
+    out = eager.reduce_residual(parts, res)
+    assert out[0, 0].item() == 1.0 + 2.0 ** -30
+    assert out[0, 1].item() == 1.0                      # ((2^53 + 1) - 2^53) + 1 with the first sum tying to 2^53
+    assert bits_equal(out, parts.sum(dim=0) + res)
+    # the normed row: double * fp32 reciprocal RMS computed from float(x)^2
+    x = torch.tensor([[3.0, 4.0]], dtype=torch.float64)
+    g = torch.tensor([2.0, 0.5], dtype=torch.float64)
+    y = eager.rmsnorm(x, g, 0.0)
+    rs = 1.0 / math.sqrt(12.5)
+    assert y.dtype == torch.float64
+    assert abs(y[0, 0].item() - 6.0 * rs) < 1e-6 and abs(y[0, 1].item() - 2.0 * rs) < 1e-6
+    assert y[0, 0].item() == 2.0 * (3.0 * float(torch.rsqrt(torch.tensor(12.5, dtype=torch.float32))))

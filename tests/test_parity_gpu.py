@@ -528,3 +528,28 @@ def test_traffic_skeleton_touches_every_byte_once(cuda_device, n, tokens, hidden
             assert torch.equal(q.reshape(tokens, -1), x[..., 0] ^ x[..., 1] ^ x[..., 2] ^ x[..., 3])
         else:
             assert torch.equal(q.reshape(tokens, -1, 2), torch.stack([x[..., 0] ^ x[..., 2], x[..., 1] ^ x[..., 3]], dim=-1))
+
+
+@pytest.mark.parametrize("n,tokens,hidden", [(2, 33, 1024), (4, 129, 2048), (8, 7, 258), (8, 300, 2), (4, 1000, 1536)])
+def test_doubles(cuda_device, n, tokens, hidden):
+    """double rows (the reference's dtype macro admits them, src/ops/all_reduce_fusion.cpp:29-33): the sum,
+    the residual add and the scaling are done in double as eager does for double tensors; only the mean of
+    squares is fp32 (test/test_all_reduce_fusion.py:25).  residual_out bit-exact, normed rows bit-identical
+    to the composition for a reciprocal RMS within 4 fp32 ulps."""
+    p, r, g = eager.make_inputs(n, tokens, hidden, torch.float64, 1.0, seed=600 + n)
+    assert p.dtype == torch.float64 and (p.view(torch.int64) & 0xFFFFFFF).ne(0).any()   # real doubles, not widened floats
+    _case("f64", p, r, g, 1e-6, "none")
+    _case("f64 table", p, r, g, 1e-6, "none", use_table=True, rank=1)
+
+
+def test_doubles_limits(cuda_device):
+    p, r, g = eager.make_inputs(2, 4, 256, torch.float64, 1.0, seed=1)
+    with pytest.raises(_capi.TdeError) as ei:
+        run_hip(p, r, g, 1e-6, "fp8_token")
+    assert ei.value.status == _capi.EQUANT
+    with pytest.raises(_capi.TdeError) as ei:
+        run_hip(p, r, g, 1e-6, "none", algo=_capi.ALGO_STAGED)
+    assert ei.value.status == _capi.EALGO
+    with pytest.raises(_capi.TdeError) as ei:
+        run_hip(p, r, g, 1e-6, "none", calls=[(("traffic",), 0)])
+    assert ei.value.status == _capi.EDTYPE

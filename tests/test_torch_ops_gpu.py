@@ -16,15 +16,16 @@ def tde(cuda_device):
     return m
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
 @pytest.mark.parametrize("tokens", [129, 128])
 def test_reference_call_sequence(tde, cuda_device, dtype, tokens):
     world_size, hidden, eps, rank = 4, 1024, 1e-6, 1
     print("case call-sequence", dtype, tokens, flush=True)
     g = torch.Generator().manual_seed(tokens)
-    allreduce_in = torch.randn((world_size, tokens, hidden), generator=g).to(dtype)
-    residual_in = torch.randn((tokens, hidden), generator=g).to(dtype)
-    gamma = torch.randn((hidden,), generator=g).to(dtype)
+    wide = torch.float64 if dtype == torch.float64 else torch.float32
+    allreduce_in = torch.randn((world_size, tokens, hidden), generator=g, dtype=wide).to(dtype)
+    residual_in = torch.randn((tokens, hidden), generator=g, dtype=wide).to(dtype)
+    gamma = torch.randn((hidden,), generator=g, dtype=wide).to(dtype)
     want = eager.reduce_rms(allreduce_in, residual_in, gamma, eps)
 
     tde.setup_env(rank, world_size)

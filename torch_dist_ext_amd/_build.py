@@ -22,7 +22,7 @@ HIP_LIB = os.path.join(PKG_DIR, "libtde_hip.so")
 TORCH_LIB = os.path.join(PKG_DIR, "libtorch_dist_ext.so")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
-HIP_SOURCES = ["tde_abi.hip", "tde_rows_bf16.hip", "tde_rows_f16.hip", "tde_rows_f32.hip", "tde_probe.hip"]
+HIP_SOURCES = ["tde_abi.hip", "tde_rows_bf16.hip", "tde_rows_f16.hip", "tde_rows_f32.hip", "tde_rows_f64.hip", "tde_probe.hip"]
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     # keep fp32 arithmetic scalar: packed fp32 forms are not used on this hardware pool
@@ -53,7 +53,7 @@ def build_hip(verbose=False):
             print(out)
         return obj
 
-    with ThreadPoolExecutor(max_workers=5) as pool:
+    with ThreadPoolExecutor(max_workers=6) as pool:
         objs = list(pool.map(compile_one, HIP_SOURCES))
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", HIP_LIB] + objs)
     return HIP_LIB

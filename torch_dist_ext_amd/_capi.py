@@ -11,7 +11,7 @@ MAX_RANKS = 16
 QUANT_GROUP = 128
 
 OK, EINVAL, ENRANKS, EDTYPE, ESHAPE, EHIDDEN, EALIGN, EQUANT, EALGO, EHIP, ERANK, ENOMEM = range(12)
-BF16, F16, F32 = 0, 1, 2
+BF16, F16, F32, F64 = 0, 1, 2, 3
 QUANT_NONE, QUANT_FP8_TOKEN, QUANT_FP8_GROUP, QUANT_INT8_TOKEN, QUANT_FP8_STATIC = 0, 1, 2, 3, 4
 ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, ALGO_STAGED_OWNED = 0, 1, 2, 3
 

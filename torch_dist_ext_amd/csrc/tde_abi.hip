@@ -23,6 +23,7 @@ int elem_bytes(int dtype) {
     case TDE_BF16:
     case TDE_F16: return 2;
     case TDE_F32: return 4;
+    case TDE_F64: return 8;
     }
     return 0;
 }
@@ -50,6 +51,10 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     if (p->quant == TDE_QUANT_FP8_STATIC && !(p->static_scale > 0.0f && p->static_scale <= 3.0e38f)) return TDE_EQUANT;
     if (p->quant == TDE_QUANT_FP8_GROUP && p->hidden % TDE_QUANT_GROUP != 0) return TDE_EQUANT;
     if (p->algo < TDE_ALGO_AUTO || p->algo > TDE_ALGO_STAGED_OWNED) return TDE_EALGO;
+    if (p->dtype == TDE_F64) { // doubles: the fused kernel only, and no quantized output
+        if (p->quant != TDE_QUANT_NONE) return TDE_EQUANT;
+        if (p->algo == TDE_ALGO_STAGED || p->algo == TDE_ALGO_STAGED_OWNED) return TDE_EALGO;
+    }
     const int vec = 16 / eb;
     const int64_t nvec = p->hidden / vec;
     if (nvec > kMaxBlock) return TDE_EHIDDEN; // as the reference: one 16-byte vector per thread, 1024 threads
@@ -70,6 +75,7 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
         vpt = 4;
     }
     if (g_force_vpt == 1 || g_force_vpt == 2 || g_force_vpt == 4) vpt = g_force_vpt;
+    if (p->dtype == TDE_F64) vpt = 1;
     const int64_t lanes = (nvec + vpt - 1) / vpt;
     const int tpr = (int)((lanes + 63) / 64 * 64);
     int rpb = 256 / tpr; // pack short rows so a workgroup has at least four wavefronts
@@ -140,9 +146,9 @@ const char *tde_status_string(int status) {
     case TDE_OK: return "ok";
     case TDE_EINVAL: return "invalid argument (null pointer or malformed struct)";
     case TDE_ENRANKS: return "nranks must be 2, 4 or 8";
-    case TDE_EDTYPE: return "unsupported dtype (bf16, f16, f32)";
+    case TDE_EDTYPE: return "unsupported dtype (bf16, f16, f32, f64)";
     case TDE_ESHAPE: return "bad shape: hidden*elem_size must be a positive multiple of 16 bytes, tokens >= 0";
-    case TDE_EHIDDEN: return "hidden too large for the one-pass row kernel (max 1024 16-byte vectors per row: 8192 bf16/f16, 4096 f32)";
+    case TDE_EHIDDEN: return "hidden too large for the one-pass row kernel (max 1024 16-byte vectors per row: 8192 bf16/f16, 4096 f32, 2048 f64)";
     case TDE_EALIGN: return "buffer not 16-byte aligned";
     case TDE_EQUANT: return "bad quant mode, per-group quant with hidden not a multiple of 128, or static scale not > 0";
     case TDE_EALGO: return "bad algorithm, or staged algorithm without a stage buffer";
@@ -274,6 +280,7 @@ int run_phases(const tde_problem *p, const tde_buffers *b, void *hip_stream, int
 
     int n = p->nranks;
     hipError_t e = hipSuccess;
+    if (traffic && p->dtype == TDE_F64) return TDE_EDTYPE;
     if (traffic) {
         const int code_bytes = quant ? (elem_bytes(p->dtype) == 4 ? 4 : 8) : 0;
         e = tde::launch_traffic(n, g.vpt, code_bytes, wn, a, g, (uint32_t)g.nvec * 16u, stream);
@@ -307,6 +314,7 @@ int run_phases(const tde_problem *p, const tde_buffers *b, void *hip_stream, int
     case TDE_BF16: e = tde::launch_rows_bf16(n, g.vpt, p->quant, wn, a, g, stream); break;
     case TDE_F16: e = tde::launch_rows_f16(n, g.vpt, p->quant, wn, a, g, stream); break;
     case TDE_F32: e = tde::launch_rows_f32(n, g.vpt, p->quant, wn, a, g, stream); break;
+    case TDE_F64: e = tde::launch_rows_f64(n, a, g, stream); break;
     }
     if (e != hipSuccess) return hip_fail(e);
     return TDE_OK;

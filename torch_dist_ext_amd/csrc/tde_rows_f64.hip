@@ -1,0 +1,111 @@
+// Rows of doubles.  The reference's dtype dispatch admits double (src/ops/all_reduce_fusion.cpp:29-33, two
+// elements per 16-byte vector); what must come out is what its torch-eager composition computes for double
+// tensors (test/test_all_reduce_fusion.py:23-28,75):
+//   x   = ((0 + p_0) + ... + p_{N-1}) + residual_in        all in double, rank order          -> residual_out
+//   rs  = 1 / sqrt( sum(float(x)^2) / H + eps )             fp32: RMSNorm.forward squares x.float()
+//   y   = gamma * (x * double(rs))                          double                              -> norm_out
+// No quantized output for this type.  One 16-byte vector per thread, the row kernel's geometry.
+#include <hip/hip_runtime.h>
+
+#include "tde_rows.h"
+
+namespace tde {
+
+__device__ __forceinline__ void unpack_f64(u32x4 raw, double (&d)[2]) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t lo = raw[2 * i], hi = raw[2 * i + 1]; // copied to scalars before the bit cast
+        const uint64_t w = ((uint64_t)hi << 32) | lo;
+        d[i] = __builtin_bit_cast(double, w);
+    }
+}
+
+__device__ __forceinline__ u32x4 pack_f64(const double (&d)[2]) {
+    u32x4 raw;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint64_t w = __builtin_bit_cast(uint64_t, d[i]);
+        raw[2 * i] = (uint32_t)w;
+        raw[2 * i + 1] = (uint32_t)(w >> 32);
+    }
+    return raw;
+}
+
+template <int N>
+__global__ void __launch_bounds__(1024) row_kernel_f64(const RowArgs a) {
+    __shared__ float lds_sum[2][kMaxWavesPerBlock];
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid >> 6;
+    const int tpr = a.threads_per_row;
+    const int waves_per_row = tpr >> 6;
+    const int group = __builtin_amdgcn_readfirstlane(tid / tpr);
+    const int t = tid - group * tpr;
+    const int first_wave = group * waves_per_row;
+    const uint32_t row_bytes = (uint32_t)a.hidden * 8u;
+    const uint32_t off = (uint32_t)t * 16u;
+
+    const void *part[N];
+#pragma unroll
+    for (int r = 0; r < N; ++r) part[r] = a.part[r];
+    if (a.table != nullptr) {
+#pragma unroll
+        for (int r = 0; r < N; ++r) {
+            const void *from_table = a.table[r];
+            part[r] = (part[r] != nullptr) ? part[r] : from_table;
+        }
+    }
+    const rsrc_t gamma_rsrc = row_rsrc(a.gamma, 0, row_bytes);
+
+    const int64_t row_stride = (int64_t)gridDim.x * a.rows_per_block;
+    int parity = 0;
+    for (int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block; row0 < a.tokens; row0 += row_stride, parity ^= 1) {
+        const int64_t row = row0 + group;
+        const uint32_t bytes = (row < a.tokens) ? row_bytes : 0u;
+        const int64_t row_byte = row * (int64_t)row_bytes;
+        u32x4 praw[N];
+#pragma unroll
+        for (int r = 0; r < N; ++r) praw[r] = rsrc_load16(row_rsrc(part[r], row_byte, bytes), off);
+        const u32x4 rraw = rsrc_load16(row_rsrc(a.residual_in, row_byte, bytes), off);
+        const u32x4 graw = __builtin_amdgcn_raw_buffer_load_b128(gamma_rsrc, (int)off, 0, kAuxDefault);
+
+        double acc[2] = {0.0, 0.0};
+#pragma unroll
+        for (int r = 0; r < N; ++r) {
+            double p[2];
+            unpack_f64(praw[r], p);
+            acc[0] += p[0];
+            acc[1] += p[1];
+        }
+        double res[2], x[2];
+        unpack_f64(rraw, res);
+        x[0] = acc[0] + res[0];
+        x[1] = acc[1] + res[1];
+        rsrc_store16(row_rsrc(a.residual_out, row_byte, bytes), off, pack_f64(x));
+
+        const float f0 = (float)x[0], f1 = (float)x[1];
+        float sumsq = f0 * f0;
+        sumsq += f1 * f1;
+        sumsq = row_reduce<OpSum>(sumsq, lds_sum[parity], wave, lane, first_wave, waves_per_row);
+        const float rs = 1.0f / __builtin_sqrtf(sumsq / a.hidden_f + a.eps);
+
+        double g[2], y[2];
+        unpack_f64(graw, g);
+        y[0] = g[0] * (x[0] * (double)rs);
+        y[1] = g[1] * (x[1] * (double)rs);
+        rsrc_store16(row_rsrc(a.norm_out, row_byte, bytes), off, pack_f64(y));
+    }
+}
+
+hipError_t launch_rows_f64(int n, const RowArgs &a, const Geometry &g, hipStream_t s) {
+    const dim3 grid((unsigned)g.grid), block((unsigned)g.block_threads);
+    switch (n) {
+    case 2: hipLaunchKernelGGL((row_kernel_f64<2>), grid, block, 0, s, a); break;
+    case 4: hipLaunchKernelGGL((row_kernel_f64<4>), grid, block, 0, s, a); break;
+    case 8: hipLaunchKernelGGL((row_kernel_f64<8>), grid, block, 0, s, a); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+} // namespace tde

@@ -40,7 +40,8 @@ int32_t dtype_code(const Tensor &t) {
     case at::kBFloat16: return TDE_BF16;
     case at::kHalf: return TDE_F16;
     case at::kFloat: return TDE_F32;
-    default: TORCH_CHECK(false, "torch_dist_ext: unsupported dtype ", t.scalar_type(), " (bf16, fp16, fp32)");
+    case at::kDouble: return TDE_F64;
+    default: TORCH_CHECK(false, "torch_dist_ext: unsupported dtype ", t.scalar_type(), " (bf16, fp16, fp32, fp64)");
     }
     return -1;
 }
