@@ -168,3 +168,31 @@ def test_slot_alias_keeps_the_workspace_alive(tde, cuda_device):
     gc.collect()
     with pytest.raises(RuntimeError, match="not a pointer table handed out"):
         tde.allreduce_rms_fusion_impl(0, 2, ref, ref, g, torch.empty_like(ref), out, 1e-6, table)
+
+
+def test_ops_under_default_torch_compile(tde, cuda_device):
+    """The custom ops inside a graph compiled with torch's default backend, which generates the surrounding
+    elementwise code itself (skipped where that backend cannot build on the host)."""
+    pytest.importorskip("triton")
+    from torch._dynamo.exc import BackendCompilerFailed
+    world_size, tokens, hidden, eps, rank = 2, 16, 1024, 1e-6, 0
+    p, r, g = eager.make_inputs(world_size, tokens, hidden, torch.bfloat16, 1.0, seed=52)
+    tde.setup_env(rank, world_size, max_size_in_bytes=tokens * hidden * 2)
+    tde.set_peer_partial(1, p[1].to(cuda_device))
+    x, rd, gd = p[0].to(cuda_device), r.to(cuda_device), g.to(cuda_device)
+    ws = tde.get_workspace(x)
+
+    def step(x, rd, gd, ws):
+        q, s, ro, _ = torch.ops.torch_dist_ext.allreduce_rms_quant(rank, world_size, x, rd, gd, eps, ws,
+                                                                    tde.QUANT_FP8_TOKEN, False)
+        return q.float() * s.unsqueeze(-1), ro.float() + 1
+
+    try:
+        deq, ro1 = torch.compile(step, fullgraph=True)(x, rd, gd, ws)
+    except BackendCompilerFailed as e:   # the code generator, not this library
+        pytest.skip("default torch.compile backend unavailable here: %s" % str(e)[:200])
+    torch.cuda.synchronize()
+    want = eager.reduce_rms(p, r, g, eps, "fp8_token")
+    assert torch.equal(ro1.cpu(), want["residual_out"].float() + 1)
+    e_deq, e_ro1 = step(x, rd, gd, ws)
+    assert torch.equal(deq, e_deq) and torch.equal(ro1, e_ro1)
