@@ -119,7 +119,8 @@ typedef struct tde_plan_out {
     int32_t vecs_per_thread; /* 16-byte vectors each thread owns per row */
     int32_t rows_per_block;  /* rows a workgroup processes side by side (one wave group per row) */
     int32_t grid_blocks;     /* workgroups launched for the row kernel */
-    int32_t reserved;
+    int32_t xcd_chunk;       /* row groups each XCD takes in a row: workgroup b of every 8*xcd_chunk takes row group
+                                (b % 8) * xcd_chunk + b / 8 of that span (1 = launch order) */
     int64_t algorithmic_bytes; /* (N+1)*T*H*e + H*e + T*H*e + OUT, OUT as documented for the quant mode */
     int64_t scale_elems;       /* number of fp32 scales written */
 } tde_plan_out;

@@ -75,6 +75,11 @@ def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, wri
         d_table = torch.tensor(ptrs, dtype=torch.int64, device=dev)
         table = d_table.data_ptr()
         ptrs = [p if r == rank else None for r, p in enumerate(ptrs)]
+    # Every output starts as 0xFF bytes (NaN in every float type): a row the kernels skip cannot pass for
+    # a result left behind in recycled memory.
+    for t in (d_res_out, d_norm, d_q, d_scale):
+        if t is not None:
+            t.view(torch.uint8).fill_(0xFF)
     stream = torch.cuda.current_stream(dev).cuda_stream
     for phases, call_rank in (calls or [(("reduce", "norm"), rank)]):
         prob = _capi.make_problem(DTYPE_CODE[dtype], n, T, H, eps, quant=qm, algo=algo, write_norm=int(bool(write_norm)),

@@ -553,3 +553,26 @@ def test_doubles_limits(cuda_device):
     with pytest.raises(_capi.TdeError) as ei:
         run_hip(p, r, g, 1e-6, "none", calls=[(("traffic",), 0)])
     assert ei.value.status == _capi.EDTYPE
+
+
+@pytest.mark.parametrize("tokens", [1, 7, 63, 64, 65, 127, 128, 129, 255, 257, 1000, 1029])
+@pytest.mark.parametrize("n", [4, 8])
+def test_row_mapping_covers_every_row_once(cuda_device, n, tokens):
+    """Workgroups take row groups in XCD-sized chunks (groups of 64 or 128 workgroups, launch order in the
+    tail): with every grid size around those group sizes, and with a capped grid that comes round again,
+    each row is produced exactly once (outputs start as NaN bytes; the traffic skeleton's exclusive-or
+    output is checked the same way)."""
+    p, r, g = eager.make_inputs(n, tokens, 512, torch.bfloat16, 1.0, seed=tokens)
+    want = eager.reduce_rms(p, r, g, 1e-6, "fp8_token")
+    for grid in (0, 96, 200):
+        _capi.tune_override(0, 0, grid)
+        try:
+            got = run_hip(p, r, g, 1e-6, "fp8_token")
+            sk = run_hip(p, r, g, 1e-6, "fp8_token", write_norm=False, calls=[(("traffic",), 0)])
+        finally:
+            _capi.tune_override(0, 0, 0)
+        check_against_oracle(got, want, "fp8_token", gamma=g, eps=1e-6)
+        x = r.contiguous().view(torch.int32).clone()
+        for k in range(n):
+            x ^= p[k].contiguous().view(torch.int32)
+        assert torch.equal(sk["residual_out"].view(torch.int32), x)

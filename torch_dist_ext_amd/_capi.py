@@ -44,7 +44,7 @@ class PlanOut(ctypes.Structure):
     _fields_ = [
         ("algo", ctypes.c_int32), ("reference_algo", ctypes.c_int32), ("vec_elems", ctypes.c_int32),
         ("block_threads", ctypes.c_int32), ("vecs_per_thread", ctypes.c_int32), ("rows_per_block", ctypes.c_int32),
-        ("grid_blocks", ctypes.c_int32), ("reserved", ctypes.c_int32), ("algorithmic_bytes", ctypes.c_int64),
+        ("grid_blocks", ctypes.c_int32), ("xcd_chunk", ctypes.c_int32), ("algorithmic_bytes", ctypes.c_int64),
         ("scale_elems", ctypes.c_int64),
     ]
 

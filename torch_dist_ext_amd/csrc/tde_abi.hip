@@ -96,6 +96,9 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
         geo->rows_per_block = rpb;
         geo->block_threads = tpr * rpb;
         geo->grid = grid;
+        // Row groups per XCD chunk of the row mapping (tde_rows.h: xcd_chunked_block); 16 measured best with 8
+        // partials, 8 with 4.
+        geo->xcd_chunk = (p->dtype == TDE_F64) ? 1 : (p->nranks >= 8 ? 16 : 8);
     }
     return TDE_OK;
 }
@@ -216,6 +219,7 @@ int tde_plan(const tde_problem *problem, tde_plan_out *plan) {
     plan->vecs_per_thread = g.vpt;
     plan->rows_per_block = g.rows_per_block;
     plan->grid_blocks = (int32_t)g.grid;
+    plan->xcd_chunk = g.xcd_chunk;
     plan->algorithmic_bytes = algorithmic_bytes(problem, &plan->scale_elems);
     return TDE_OK;
 }
@@ -274,6 +278,7 @@ int run_phases(const tde_problem *p, const tde_buffers *b, void *hip_stream, int
     a.nvec = g.nvec;
     a.threads_per_row = g.threads_per_row;
     a.rows_per_block = g.rows_per_block;
+    a.xcd_chunk = g.xcd_chunk;
     a.eps = p->eps;
     a.hidden_f = (float)p->hidden;
     a.static_scale = p->static_scale;
