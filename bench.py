@@ -22,7 +22,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 
 # HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs summarized under
 # profiles/ (scaled by the plain-copy calibration described there); None where not collected.
-TRAFFIC_BYTES = {"c2": 11655354, "c3": 352692441, "c4": 765430448, "c5": 2182061403}
+TRAFFIC_BYTES = {"c2": 11655354, "c3": 352644601, "c4": 765430448, "c5": 2182061403}
 
 BENCH_CONFIGS = {
     # name: (N, T, H, dtype, sigma, eps, quant)
