@@ -515,6 +515,7 @@ struct ReduceSpan {
     int64_t first_row;
     int64_t row_step;
     int64_t spans_per_row;
+    uint32_t xcd_chunk; // spans each XCD takes in a row (xcd_chunked_block); 16 over whole tensors, 1 for single rows
 };
 
 template <class E, int N, int U>
@@ -531,8 +532,9 @@ __global__ void __launch_bounds__(256) reduce_kernel(const RowArgs a, const Redu
             part[r] = (part[r] != nullptr) ? part[r] : from_table;
         }
     }
-    const int64_t k = (int64_t)blockIdx.x / sp.spans_per_row;
-    const int64_t in_row = ((int64_t)blockIdx.x - k * sp.spans_per_row) * SPAN;
+    const int64_t bid = xcd_chunked_block(blockIdx.x, gridDim.x, sp.xcd_chunk);
+    const int64_t k = bid / sp.spans_per_row;
+    const int64_t in_row = (bid - k * sp.spans_per_row) * SPAN;
     const int64_t base = (sp.first_row + k * sp.row_step) * sp.row_bytes + in_row;
     const int64_t left = sp.row_bytes - in_row;
     const uint32_t bytes = left < (int64_t)SPAN ? (uint32_t)left : SPAN;
@@ -635,7 +637,7 @@ template <class E, int N, int U>
 hipError_t launch_reduce_nu(const RowArgs &a, int64_t row_bytes, int64_t first_row, int64_t row_step, int64_t rows,
                             hipStream_t s) {
     constexpr int64_t span = 256 * U * 16;
-    ReduceSpan sp{row_bytes, first_row, row_step, (row_bytes + span - 1) / span};
+    ReduceSpan sp{row_bytes, first_row, row_step, (row_bytes + span - 1) / span, rows == 1 ? 16u : 1u};
     const int64_t blocks = rows * sp.spans_per_row;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffff) return hipErrorInvalidValue; // grid dimension limit
