@@ -227,10 +227,30 @@ def main():
                      "traffic_only_us": floor_us,
                      "traffic_only_frac": (bytes_per_launch / (floor_us * 1e-6) / 1e9 / HBM_PEAK_GBS) if floor_us else None},
     }
+    # The device's practical streaming rates, measured now (tde_probe_stream: 1 GiB per launch, four buffers
+    # in rotation): what reads alone, writes alone and a plain copy reach on this box.
+    del sets, calls, call_refs
+    torch.cuda.empty_cache()
+    gib = 1 << 30
+    bufs = [torch.empty(gib, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(4)]
+    rates = {}
+    for mode, name, moved in ((0, "read_only_GBs", gib), (1, "write_only_GBs", gib), (2, "copy_GBs", 2 * gib)):
+        for i in range(3):
+            _capi.probe_stream(bufs[i % 4].data_ptr(), bufs[(i + 1) % 4].data_ptr(), gib, mode, stream.cuda_stream)
+        torch.cuda.synchronize(dev)
+        ev4 = torch.cuda.Event(enable_timing=True)
+        ev5 = torch.cuda.Event(enable_timing=True)
+        ev4.record(stream)
+        for i in range(12):
+            _capi.probe_stream(bufs[i % 4].data_ptr(), bufs[(i + 1) % 4].data_ptr(), gib, mode, stream.cuda_stream)
+        ev5.record(stream)
+        torch.cuda.synchronize(dev)
+        rates[name] = moved / (ev4.elapsed_time(ev5) * 1e-3 / 12) / 1e9
+    del bufs
     info = _capi.device_info()
     out["device"] = {"name": torch.cuda.get_device_properties(dev).name, "compute_units": info.compute_units,
                      "memory_clock_khz": info.memory_clock_khz, "memory_bus_bits": info.memory_bus_bits,
-                     "hbm_bytes": info.total_memory_bytes,
+                     "hbm_bytes": info.total_memory_bytes, **rates,
                      # transfers per reported memory clock that the published 8 TB/s corresponds to
                      "peak_transfers_per_clock": (HBM_PEAK_GBS * 1e9 * 8 / (info.memory_bus_bits * info.memory_clock_khz * 1e3)
                                                   if info.memory_bus_bits and info.memory_clock_khz else None)}

@@ -168,6 +168,11 @@ int tde_tune_override(int32_t vecs_per_thread, int32_t rows_per_block, int32_t m
    measuring the device's practical streaming ceiling.  No counterpart in the reference. */
 int tde_probe_copy(void *dst, const void *src, int64_t bytes, void *hip_stream);
 
+/* Measurement aid: the device's practical streaming rates.  mode 0 reads `bytes` from src (dst, at least 16
+   bytes, is not written for any realistic data), 1 writes `bytes` to dst (src is not read), 2 copies; one
+   workgroup per 4 KiB, no loop.  `bytes` a multiple of 16.  No counterpart in the reference. */
+int tde_probe_stream(void *dst, const void *src, int64_t bytes, int32_t mode, void *hip_stream);
+
 /* Measurement aid: the memory traffic of tde_reduce_rms for the same problem and buffers with the arithmetic
    removed -- same workgroups, lane mapping, load order and cache policies, every input byte read and every
    output byte (scales excepted) written once, contents meaningless.  OVERWRITES residual_out, norm_out and

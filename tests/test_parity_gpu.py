@@ -576,3 +576,23 @@ def test_row_mapping_covers_every_row_once(cuda_device, n, tokens):
         for k in range(n):
             x ^= p[k].contiguous().view(torch.int32)
         assert torch.equal(sk["residual_out"].view(torch.int32), x)
+
+
+def test_stream_probe(cuda_device):
+    n = 1 << 20
+    src = torch.empty(n + 16, dtype=torch.uint8, device=cuda_device).random_(0, 255)
+    dst = torch.zeros(n + 16, dtype=torch.uint8, device=cuda_device)
+    st = torch.cuda.current_stream().cuda_stream
+    _capi.probe_stream(dst.data_ptr(), src.data_ptr(), n - 48, 2, st)          # copy, ragged last workgroup
+    torch.cuda.synchronize()
+    assert torch.equal(dst[:n - 48], src[:n - 48]) and int(dst[n - 48:].sum()) == 0
+    dst.zero_()
+    _capi.probe_stream(dst.data_ptr(), src.data_ptr(), n, 0, st)               # read only: nothing written
+    torch.cuda.synchronize()
+    assert int(dst.sum()) == 0
+    _capi.probe_stream(dst.data_ptr(), src.data_ptr(), n, 1, st)               # write only: every vector written
+    torch.cuda.synchronize()
+    words = dst[:n].view(torch.int32).view(-1, 4)
+    assert bool((words[:, 2] == 0x9e3779b9 - (1 << 32)).all()) and int(dst[n:].sum()) == 0
+    with pytest.raises(_capi.TdeError):
+        _capi.probe_stream(dst.data_ptr(), src.data_ptr(), n, 3, st)

@@ -18,7 +18,7 @@ ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, ALGO_STAGED_OWNED = 0, 1, 2, 3
 # Every symbol include/tde_abi.h declares.
 EXPORTS = (
     "tde_abi_version", "tde_status_string", "tde_last_hip_error", "tde_plan", "tde_reduce_rms", "tde_stage_reduce", "tde_stage_norm",
-    "tde_tune_override", "tde_probe_copy", "tde_probe_rows", "tde_device_info",
+    "tde_tune_override", "tde_probe_copy", "tde_probe_stream", "tde_probe_rows", "tde_device_info",
     "tde_workspace_create", "tde_workspace_destroy", "tde_workspace_slot", "tde_workspace_stage",
     "tde_workspace_slot_bytes", "tde_workspace_nranks", "tde_workspace_fill_table",
 )
@@ -88,6 +88,8 @@ def load():
     lib.tde_tune_override.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
     lib.tde_probe_copy.restype = ctypes.c_int
     lib.tde_probe_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+    lib.tde_probe_stream.restype = ctypes.c_int
+    lib.tde_probe_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p]
     lib.tde_device_info.restype = ctypes.c_int
     lib.tde_device_info.argtypes = [ctypes.POINTER(DeviceInfo)]
     lib.tde_workspace_create.restype = ctypes.c_int
@@ -159,6 +161,11 @@ def device_info():
     out = DeviceInfo()
     check(load().tde_device_info(ctypes.byref(out)))
     return out
+
+
+def probe_stream(dst, src, nbytes, mode, stream=None):
+    """tde_probe_stream: mode 0 read-only, 1 write-only, 2 copy."""
+    check(load().tde_probe_stream(dst, src, nbytes, mode, stream))
 
 
 def probe_copy(dst, src, nbytes, stream=None):
