@@ -354,22 +354,35 @@ def test_static_scale_is_validated(cuda_device):
         assert e.value.status == _capi.EQUANT
 
 
-def test_hip_graph_replays_match_eager(cuda_device):
-    """The launch allocates nothing and synchronizes nothing, so it can be captured.  Replays are checked
-    against eager launches, with new input contents and eager work between the replays."""
+@pytest.mark.parametrize("algo", [_capi.ALGO_FUSED, _capi.ALGO_STAGED, _capi.ALGO_STAGED_OWNED])
+def test_hip_graph_replays_match_eager(cuda_device, algo):
+    """The launch allocates nothing and synchronizes nothing, so it can be captured (the staged algorithms:
+    both launches in one graph).  Replays are checked against eager launches, with new input contents and
+    eager work between the replays."""
     dev = cuda_device
     n, t, h = 8, 128, 4096
+    stage = torch.empty((t, h), dtype=torch.bfloat16, device=dev) if algo != _capi.ALGO_FUSED else None
     parts = [torch.empty((t, h), dtype=torch.bfloat16, device=dev) for _ in range(n)]
     res = torch.empty((t, h), dtype=torch.bfloat16, device=dev)
     gamma = torch.empty((h,), dtype=torch.bfloat16, device=dev)
     outs = {k: torch.empty((t, h), dtype=torch.bfloat16, device=dev) for k in ("res_out", "norm")}
     q = torch.empty((t, h), dtype=torch.uint8, device=dev)
     sc = torch.empty((t,), dtype=torch.float32, device=dev)
-    prob = _capi.make_problem(_capi.BF16, n, t, h, 1e-5, quant=_capi.QUANT_FP8_TOKEN, write_norm=1)
+    prob = _capi.make_problem(_capi.BF16, n, t, h, 1e-5, quant=_capi.QUANT_FP8_TOKEN, write_norm=1, algo=algo)
 
     def launch(stream):
+        if algo == _capi.ALGO_STAGED_OWNED:       # all N ranks' shares, then the norm: the whole two-shot
+            for k in range(n):
+                pk = _capi.make_problem(_capi.BF16, n, t, h, 1e-5, quant=_capi.QUANT_FP8_TOKEN, write_norm=1, algo=algo, rank=k)
+                _capi.reduce_rms(pk, [p.data_ptr() for p in parts], None, None, None, stage=stage.data_ptr(), stream=stream,
+                                 phases=("reduce",))
+            _capi.reduce_rms(prob, [None] * n, res.data_ptr(), outs["res_out"].data_ptr(), gamma.data_ptr(),
+                             norm_out=outs["norm"].data_ptr(), q_out=q.data_ptr(), scale_out=sc.data_ptr(),
+                             stage=stage.data_ptr(), stream=stream, phases=("norm",))
+            return
         _capi.reduce_rms(prob, [p.data_ptr() for p in parts], res.data_ptr(), outs["res_out"].data_ptr(), gamma.data_ptr(),
-                         norm_out=outs["norm"].data_ptr(), q_out=q.data_ptr(), scale_out=sc.data_ptr(), stream=stream)
+                         norm_out=outs["norm"].data_ptr(), q_out=q.data_ptr(), scale_out=sc.data_ptr(),
+                         stage=stage.data_ptr() if stage is not None else None, stream=stream)
 
     def fill(seed):
         cp, cr, cg = eager.make_inputs(n, t, h, torch.bfloat16, 0.5, seed=seed)
