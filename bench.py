@@ -91,7 +91,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (one rank's stage with N local partial buffers); "
-              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+              "--gpus %d with WORLD_SIZE=%s is not supported" % (args.gpus, os.environ.get("WORLD_SIZE", "1")), file=sys.stderr)
         sys.exit(2)
 
     import torch
