@@ -175,6 +175,8 @@ def test_ops_under_default_torch_compile(tde, cuda_device):
     elementwise code itself (skipped where that backend cannot build on the host)."""
     pytest.importorskip("triton")
     from torch._dynamo.exc import BackendCompilerFailed
+    import torch._inductor.config as inductor_config
+    inductor_config.compile_threads = 1      # compile in this process: no pool of worker processes
     world_size, tokens, hidden, eps, rank = 2, 16, 1024, 1e-6, 0
     p, r, g = eager.make_inputs(world_size, tokens, hidden, torch.bfloat16, 1.0, seed=52)
     tde.setup_env(rank, world_size, max_size_in_bytes=tokens * hidden * 2)
