@@ -19,7 +19,9 @@ all_reduce_fusion_impl.h:26,313 are unused) and its tests assert nothing, so:
   PARITY UNPINNED by the reference: quant_fp8 / quant_int8 / quant_fp8_static.  Their definition is this build's own
            (scale = amax/448 resp. amax/127, RNE codes, clamp); they are pinned only against the
            mathematics: a textbook e4m3 encoder over all codes and midpoints, max-code and
-           half-step dequantization properties, ties-to-even for int8.
+           half-step dequantization properties, ties-to-even for int8; quant_fp8_static through
+           power-of-two scales (exact quotients -> the textbook encoder), saturation at +-448*scale and
+           bit equality with quant_fp8 when given a row's own dynamic scale.
 """
 import torch
 

@@ -145,7 +145,8 @@ def quant_from_own_norm(norm_got, quant):
     return eager.quant_int8(norm_got)
 
 
-def check_against_oracle(got, want, quant, gamma=None, eps=None, norm_ulp=2, norm_flip_frac=2e-4, scale_rtol=1e-6):
+def check_against_oracle(got, want, quant, gamma=None, eps=None, norm_ulp=None, norm_flip_frac=2e-4, scale_rtol=1e-6,
+                         strict=False):
     """Two levels.
 
     Stage-exact (needs gamma/eps and a norm_out from the kernel):
@@ -158,6 +159,9 @@ def check_against_oracle(got, want, quant, gamma=None, eps=None, norm_ulp=2, nor
       differs in its last fp32 bit; codes within one quant step; scales within scale_rtol relative,
       except rows/groups whose maximum element is one of those flipped elements (counted, and bounded
       by the number of flipped elements).
+    norm_ulp defaults to 1 for bf16 (the stated bound: normed bf16 within 1 bf16 ulp) and 2 for fp16, whose
+    second rounding can carry a first-rounding flip one step further.  strict=True (the bf16 benchmark
+    configurations) additionally demands that no scale at all is outside scale_rtol.
     Returns mismatch statistics."""
     stats = {}
     assert bits_equal(got["residual_out"], want["residual_out"]), "residual_out is not bit-exact"
@@ -185,7 +189,12 @@ def check_against_oracle(got, want, quant, gamma=None, eps=None, norm_ulp=2, nor
             assert float((got["norm_out"] - want["norm_out"]).abs().max()) <= 1e-4 * magnitude
             flipped = got["norm_out"].shape[0]
         else:
-            assert stats["norm_max_ulp"] <= norm_ulp, "norm_out off by %d ulp" % stats["norm_max_ulp"]
+            if norm_ulp is None:
+                norm_ulp = 1 if got["norm_out"].dtype == torch.bfloat16 else 2
+            assert stats["norm_max_ulp"] <= norm_ulp, (
+                "norm_out off by %d ulp (allowed %d: 1 for bf16; 2 for fp16, where a first rounding that lands on the "
+                "other side because the reciprocal RMS differs in its last fp32 bit can move the second rounding too)"
+                % (stats["norm_max_ulp"], norm_ulp))
             assert flipped / n <= norm_flip_frac, "%d of %d normed elements differ" % (flipped, n)
         if gamma is not None:
             ok, matched = norm_rows_explained(got["norm_out"], got["residual_out"], gamma, eps)
@@ -204,6 +213,10 @@ def check_against_oracle(got, want, quant, gamma=None, eps=None, norm_ulp=2, nor
         bad = int((rel > scale_rtol).sum())
         stats["scale_max_rel"] = float(rel.max()) if rel.numel() else 0.0
         stats["scale_bad"] = bad
+        if strict:
+            assert bad == 0, "%d scales differ by more than %g relative (max %g)" % (bad, scale_rtol, stats["scale_max_rel"])
+        # otherwise (fp16/fp32 rows, randomized and extreme-magnitude cases): a scale may differ only where the row's
+        # maximum is one of the elements whose rounding flipped with the last bit of the reciprocal RMS
         assert bad <= flipped, "%d scales differ by more than %g relative (max %g) with only %d flipped elements" % (
             bad, scale_rtol, stats["scale_max_rel"], flipped)
         assert stats["scale_max_rel"] <= 2.0 ** -7, "a scale is off by more than one ulp of the element type"

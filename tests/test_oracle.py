@@ -250,6 +250,52 @@ def test_int8_quant_properties_and_ties_to_even():
     assert float(ss) == 1.0 and qq.tolist() == [[127, 0, 2, 2, 0, -2, -2, 4]]
 
 
+@pytest.mark.parametrize("scale", [1.0, 0.0078125, 64.0])
+def test_static_scale_fp8_power_of_two_scales_are_the_textbook_encoder(scale):
+    """quant_fp8_static (the mode behind the reference's unused scale_factor field,
+    src/common/all_reduce_fusion_impl.h:313): with a power-of-two scale y/scale is exact, so the codes must be
+    the textbook e4m3 encoding of y/scale -- every representable value, every midpoint (ties to even) and
+    both fp32 neighbours of every midpoint."""
+    L = cport.lib()
+    finite = sorted(set(_textbook_e4m3_decode(c) for c in range(0x7F)))
+    mids = [(lo + hi) / 2 for lo, hi in zip(finite[:-1], finite[1:])]
+    near = []
+    for lo, hi, mid in zip(finite[:-1], finite[1:], mids):
+        near += [float(np.nextafter(np.float32(mid), np.float32(lo))), float(np.nextafter(np.float32(mid), np.float32(hi)))]
+    pos = torch.tensor(finite + mids + near, dtype=torch.float32)
+    x = torch.cat([pos, -pos]) * scale            # exact: scale is a power of two
+    got = eager.quant_fp8_static(x.view(1, -1), scale).view(torch.uint8).view(-1)
+    for v, c in zip((x / scale).tolist(), got.tolist()):
+        assert c == L.tdo_f32_to_e4m3(v), (v, c)
+    n = len(finite)
+    assert got[:n].tolist() == [L.tdo_f32_to_e4m3(v) for v in finite]            # representable values map to themselves
+    assert all(c & 1 == 0 for c in got[n:n + len(mids)].tolist())                # midpoints go to the even code
+
+
+def test_static_scale_fp8_saturates_and_equals_dynamic_quant_at_its_own_scale():
+    # beyond 448*scale the code saturates at the top finite code, never NaN (0x7F / 0xFF)
+    scale = 0.013
+    x = torch.tensor([[448.0 * scale * 1.001, 1e4, 3e38, -448.0 * scale * 1.001, -1e4, -3e38, 0.0, -0.0]], dtype=torch.float32)
+    q = eager.quant_fp8_static(x, scale).view(torch.uint8).view(-1).tolist()
+    assert q[:3] == [0x7E] * 3 and q[3:6] == [0xFE] * 3 and q[6] & 0x7F == 0 and q[7] & 0x7F == 0
+    # with the row's own dynamic scale (amax/448) the static mode is the dynamic mode, bit for bit
+    p, r, g = eager.make_inputs(4, 16, 512, torch.bfloat16, 1.0, seed=14)
+    y = eager.reduce_rms(p, r, g, 1e-6, "none")["norm_out"]
+    qd, sd = eager.quant_fp8(y, None)
+    for row in range(y.shape[0]):
+        qs = eager.quant_fp8_static(y[row:row + 1], float(sd[row]))
+        assert torch.equal(qs.view(torch.uint8), qd[row:row + 1].view(torch.uint8))
+    # bf16 inputs and an arbitrary scale: codes equal the C restatement's encoder applied to the fp32 quotient
+    L = cport.lib()
+    s32 = np.float32(0.0371)
+    qs = eager.quant_fp8_static(y, float(s32)).view(torch.uint8).numpy()
+    quot = np.clip(y.float().numpy() / s32, -448.0, 448.0).astype(np.float32)
+    want = np.array([L.tdo_f32_to_e4m3(float(v)) for v in quot.reshape(-1)], dtype=np.uint8).reshape(quot.shape)
+    # +0 and -0 quotients are both zero codes; the sign bit of a zero code is not part of the contract here
+    same = (qs == want) | (((qs & 0x7F) == 0) & ((want & 0x7F) == 0))
+    assert same.all()
+
+
 def test_zero_row_quantizes_to_zero_scale_and_codes():
     z = torch.zeros((2, 256), dtype=torch.bfloat16)
     for fn in (lambda y: eager.quant_fp8(y, None), lambda y: eager.quant_fp8(y, 128), eager.quant_int8):
