@@ -29,6 +29,7 @@ extern "C" {
 #define TDE_ABI_VERSION 1
 #define TDE_MAX_RANKS 16 /* array bound, as MAX_RANKS in src/ops/all_reduce_fusion.h:8 */
 #define TDE_QUANT_GROUP 128
+#define TDE_STATIC_STAGE_BYTES (32 << 20) /* stage held inside the library for tde_reduce_rms_static_stage */
 
 /* ---- status codes ------------------------------------------------------------------------- */
 typedef enum tde_status {
@@ -44,7 +45,8 @@ typedef enum tde_status {
     TDE_EALGO = 8,      /* unknown algorithm, staged algorithm without a stage buffer or with TDE_F64 */
     TDE_EHIP = 9,       /* HIP runtime error; see tde_last_hip_error() */
     TDE_ERANK = 10,     /* rank outside [0,nranks) */
-    TDE_ENOMEM = 11     /* device allocation failed */
+    TDE_ENOMEM = 11,    /* device allocation failed */
+    TDE_ETOOBIG = 12    /* tde_reduce_rms_static_stage: the rows do not fit the library's static stage */
 } tde_status;
 
 /* ---- enums ---------------------------------------------------------------------------------- */
@@ -156,6 +158,18 @@ int tde_reduce_rms(const tde_problem *problem, const tde_buffers *buffers, void 
    tde_reduce_rms with the same problem is exactly tde_stage_reduce followed by tde_stage_norm. */
 int tde_stage_reduce(const tde_problem *problem, const tde_buffers *buffers, void *hip_stream);
 int tde_stage_norm(const tde_problem *problem, const tde_buffers *buffers, void *hip_stream);
+
+/* tde_reduce_rms with the staged algorithm (TDE_ALGO_STAGED; TDE_ALGO_AUTO means the same here, any other
+   algorithm is TDE_EALGO) and the stage buffer taken from a fixed array inside the library's device image
+   instead of buffers->stage (which is ignored).  After its first call on a device (which looks the array's
+   address up) it calls no allocator and nothing that allocates: for callers that cannot allocate -- code under
+   HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+   reference, whose stage lives in the CommWorkspace allocation (src/ops/all_reduce_fusion.cpp:70-74).
+   Limit: tokens * hidden * elem_size <= TDE_STATIC_STAGE_BYTES (32 MiB, e.g. 2048 x 8192 bf16), else
+   TDE_ETOOBIG.  Every GPU the library runs on holds one copy of the array until the process ends, and every
+   call on a GPU uses that copy: calls that overlap on one GPU (different streams, different threads) race.
+   Each call overwrites the part of the array it reads, so nothing needs clearing between calls. */
+int tde_reduce_rms_static_stage(const tde_problem *problem, const tde_buffers *buffers, void *hip_stream);
 
 /* Tuning hook for sweeps and tests: force vectors-per-thread (1,2,4), rows per workgroup and a cap
    on the grid (rows beyond it are covered by a grid-stride loop).  0 restores the automatic choice

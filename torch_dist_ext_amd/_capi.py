@@ -10,7 +10,8 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libtde_hip.
 MAX_RANKS = 16
 QUANT_GROUP = 128
 
-OK, EINVAL, ENRANKS, EDTYPE, ESHAPE, EHIDDEN, EALIGN, EQUANT, EALGO, EHIP, ERANK, ENOMEM = range(12)
+OK, EINVAL, ENRANKS, EDTYPE, ESHAPE, EHIDDEN, EALIGN, EQUANT, EALGO, EHIP, ERANK, ENOMEM, ETOOBIG = range(13)
+STATIC_STAGE_BYTES = 32 << 20
 BF16, F16, F32, F64 = 0, 1, 2, 3
 QUANT_NONE, QUANT_FP8_TOKEN, QUANT_FP8_GROUP, QUANT_INT8_TOKEN, QUANT_FP8_STATIC = 0, 1, 2, 3, 4
 ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, ALGO_STAGED_OWNED = 0, 1, 2, 3
@@ -18,6 +19,7 @@ ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, ALGO_STAGED_OWNED = 0, 1, 2, 3
 # Every symbol include/tde_abi.h declares.
 EXPORTS = (
     "tde_abi_version", "tde_status_string", "tde_last_hip_error", "tde_plan", "tde_reduce_rms", "tde_stage_reduce", "tde_stage_norm",
+    "tde_reduce_rms_static_stage",
     "tde_tune_override", "tde_probe_copy", "tde_probe_stream", "tde_probe_rows", "tde_device_info",
     "tde_workspace_create", "tde_workspace_destroy", "tde_workspace_slot", "tde_workspace_stage",
     "tde_workspace_slot_bytes", "tde_workspace_nranks", "tde_workspace_fill_table",
@@ -81,7 +83,7 @@ def load():
     lib.tde_plan.argtypes = [ctypes.POINTER(Problem), ctypes.POINTER(PlanOut)]
     lib.tde_reduce_rms.restype = ctypes.c_int
     lib.tde_reduce_rms.argtypes = [ctypes.POINTER(Problem), ctypes.POINTER(Buffers), ctypes.c_void_p]
-    for fn in (lib.tde_stage_reduce, lib.tde_stage_norm, lib.tde_probe_rows):
+    for fn in (lib.tde_stage_reduce, lib.tde_stage_norm, lib.tde_probe_rows, lib.tde_reduce_rms_static_stage):
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(Problem), ctypes.POINTER(Buffers), ctypes.c_void_p]
     lib.tde_tune_override.restype = ctypes.c_int
@@ -139,7 +141,8 @@ def reduce_rms(problem, partials, residual_in, residual_out, gamma, norm_out=Non
                stage=None, partial_table=None, stream=None, phases=("reduce", "norm")):
     """tde_reduce_rms with raw device addresses (ints).  `partials` is a sequence of addresses (None
     entries are taken from partial_table).  phases=("reduce",) / ("norm",) calls tde_stage_reduce /
-    tde_stage_norm instead, phases=("traffic",) tde_probe_rows.  Raises TdeError on a non-zero status."""
+    tde_stage_norm instead, phases=("traffic",) tde_probe_rows, phases=("static_stage",)
+    tde_reduce_rms_static_stage.  Raises TdeError on a non-zero status."""
     b = Buffers()
     for r, p in enumerate(partials):
         b.partial[r] = p
@@ -148,7 +151,8 @@ def reduce_rms(problem, partials, residual_in, residual_out, gamma, norm_out=Non
     b.q_out, b.scale_out, b.stage = q_out, scale_out, stage
     lib = load()
     fn = {("reduce", "norm"): lib.tde_reduce_rms, ("reduce",): lib.tde_stage_reduce,
-          ("norm",): lib.tde_stage_norm, ("traffic",): lib.tde_probe_rows}[tuple(phases)]
+          ("norm",): lib.tde_stage_norm, ("traffic",): lib.tde_probe_rows,
+          ("static_stage",): lib.tde_reduce_rms_static_stage}[tuple(phases)]
     check(fn(ctypes.byref(problem), ctypes.byref(b), stream))
 
 

@@ -4,10 +4,16 @@
 
 #include <cstdint>
 #include <cstring>
+#include <mutex>
 #include <new>
 
 #include "tde_abi.h"
 #include "tde_rows.h"
+
+// Stage buffer of tde_reduce_rms_static_stage: part of the library's device image, one copy per GPU, held
+// until the process ends.  Host code never uses this name as an address: static_stage_ptr() asks the
+// runtime for the current device's copy once and keeps the answer.
+static __device__ __align__(256) unsigned char scratch[TDE_STATIC_STAGE_BYTES];
 
 namespace {
 
@@ -26,6 +32,28 @@ int elem_bytes(int dtype) {
     case TDE_F64: return 8;
     }
     return 0;
+}
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int static_stage_ptr(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e);
+    if (dev < 0 || dev >= kMaxDevices) return TDE_EINVAL;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_fail(e);
+        if (ptr == nullptr) return TDE_EINVAL;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return TDE_OK;
 }
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -178,6 +206,7 @@ const char *tde_status_string(int status) {
     case TDE_EHIP: return "HIP runtime error (see tde_last_hip_error)";
     case TDE_ERANK: return "rank outside [0, nranks)";
     case TDE_ENOMEM: return "device allocation failed";
+    case TDE_ETOOBIG: return "tokens*hidden*elem_size exceeds the library's static stage (TDE_STATIC_STAGE_BYTES)";
     }
     return "unknown status";
 }
@@ -373,6 +402,23 @@ int tde_stage_reduce(const tde_problem *p, const tde_buffers *b, void *hip_strea
 
 int tde_stage_norm(const tde_problem *p, const tde_buffers *b, void *hip_stream) {
     return run_phases(p, b, hip_stream, kPhaseNorm);
+}
+
+int tde_reduce_rms_static_stage(const tde_problem *p, const tde_buffers *b, void *hip_stream) {
+    if (p == nullptr || b == nullptr) return TDE_EINVAL;
+    if (p->algo != TDE_ALGO_AUTO && p->algo != TDE_ALGO_STAGED) return TDE_EALGO;
+    tde_problem staged = *p;
+    staged.algo = TDE_ALGO_STAGED;
+    const int st = validate(&staged, nullptr);
+    if (st != TDE_OK) return st;
+    // validate() has bounded hidden and checked that tokens * hidden * elem does not overflow
+    if (p->tokens * p->hidden * elem_bytes(p->dtype) > (int64_t)TDE_STATIC_STAGE_BYTES) return TDE_ETOOBIG;
+    void *stage = nullptr;
+    const int sp = static_stage_ptr(&stage);
+    if (sp != TDE_OK) return sp;
+    tde_buffers with_stage = *b;
+    with_stage.stage = stage;
+    return run_phases(&staged, &with_stage, hip_stream, kPhaseReduce | kPhaseNorm);
 }
 
 int tde_probe_rows(const tde_problem *p, const tde_buffers *b, void *hip_stream) {
