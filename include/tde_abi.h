@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define TDE_ABI_VERSION 1
+#define TDE_ABI_VERSION 2
 #define TDE_MAX_RANKS 16 /* array bound, as MAX_RANKS in src/ops/all_reduce_fusion.h:8 */
 #define TDE_QUANT_GROUP 128
 #define TDE_STATIC_STAGE_BYTES (32 << 20) /* stage held inside the library for tde_reduce_rms_static_stage */
@@ -93,6 +93,11 @@ typedef struct tde_problem {
     int64_t hidden;     /* columns per row */
     float eps;          /* added to mean(x^2) before the reciprocal square root */
     float static_scale; /* TDE_QUANT_FP8_STATIC: code = e4m3(clamp(y / static_scale, +-448)); must be > 0 and finite */
+    /* Launch-geometry overrides for sweeps and tests, per call; 0 = automatic.  The reference's launcher
+       hard-codes its geometry (impl.h:481-489) and has no counterpart. */
+    int32_t tune_vecs_per_thread; /* 1, 2 or 4 16-byte vectors per thread per row (other non-zero values: TDE_EINVAL) */
+    int32_t tune_rows_per_block;  /* rows side by side in one workgroup; ignored where it would exceed the
+                                     kernel's launch bound of 1024 / vecs_per_thread threads */
 } tde_problem;
 
 typedef struct tde_buffers {
@@ -139,8 +144,10 @@ const char *tde_status_string(int status);
 int tde_last_hip_error(void);
 
 /* Pure host: validates the problem exactly as tde_reduce_rms does and reports launch geometry and
-   algorithmic bytes.  Touches no device.  Replaces the shape/nranks asserts and the grid/block/
-   algorithm selection of allreduce_fusion_kernel_launcher (impl.h:476-498, 526-534). */
+   algorithmic bytes.  Launches nothing; the geometry is sized for the current device's compute-unit
+   count (asked once per device), or for 256 compute units where no device is present.  Replaces the
+   shape/nranks asserts and the grid/block/algorithm selection of allreduce_fusion_kernel_launcher
+   (impl.h:476-498, 526-534). */
 int tde_plan(const tde_problem *problem, tde_plan_out *plan);
 
 /* Enqueue the row kernel(s) on `hip_stream` (a hipStream_t, null = default stream) of the current
@@ -170,12 +177,6 @@ int tde_stage_norm(const tde_problem *problem, const tde_buffers *buffers, void 
    call on a GPU uses that copy: calls that overlap on one GPU (different streams, different threads) race.
    Each call overwrites the part of the array it reads, so nothing needs clearing between calls. */
 int tde_reduce_rms_static_stage(const tde_problem *problem, const tde_buffers *buffers, void *hip_stream);
-
-/* Tuning hook for sweeps and tests: force vectors-per-thread (1,2,4), rows per workgroup and a cap
-   on the grid (rows beyond it are covered by a grid-stride loop).  0 restores the automatic choice
-   for that field.  Process-wide, not thread-safe.  No counterpart in the reference, whose
-   launcher hard-codes its geometry (impl.h:481-489). */
-int tde_tune_override(int32_t vecs_per_thread, int32_t rows_per_block, int32_t max_grid);
 
 /* Calibration: enqueue a plain copy of `bytes` (multiple of 16) from src to dst on `hip_stream`.
    Known traffic (bytes read + bytes written) for scaling profiler memory counters and for

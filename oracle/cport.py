@@ -17,7 +17,7 @@ REF_LIB = os.path.join(HERE, "_ref", "libunit_ref.so")
 
 BF16, F16, F32 = 0, 1, 2
 QUANT = {"none": 0, "fp8_token": 1, "fp8_group": 2, "int8_token": 3}
-SUMSQ_F32_SEQ, SUMSQ_F64, SUMSQ_F32_PAIRWISE = 0, 1, 2
+SUMSQ_F32_SEQ, SUMSQ_F64, SUMSQ_F32_PAIRWISE, SUMSQ_TORCH = 0, 1, 2, 3
 
 _lib = None
 _ref = None
@@ -51,6 +51,8 @@ def lib():
             ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.POINTER(ctypes.c_void_p),
             ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
             ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+        L.tdo_torch_row_sum.restype = ctypes.c_float
+        L.tdo_torch_row_sum.argtypes = [ctypes.c_void_p, ctypes.c_int64]
         L.tdo_unit_test_ref.restype = ctypes.c_int
         L.tdo_unit_test_ref.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int64, ctypes.c_int64, ctypes.c_int] + \
             [ctypes.c_void_p] * 2 + [ctypes.c_float]
@@ -104,6 +106,13 @@ def reduce_rms(dtype, parts, residual, gamma, eps, quant="none", sumsq_mode=SUMS
     if qm:
         out["q"], out["scale"] = q, scale
     return out
+
+
+def torch_row_sums(a):
+    """Row sums of a C-contiguous float32 [T, n] array in the order of torch's CPU reduction (tdo_torch_row_sum)."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    L = lib()
+    return np.array([L.tdo_torch_row_sum(a[i].ctypes.data, a.shape[1]) for i in range(a.shape[0])], dtype=np.float32)
 
 
 def _unit(fn, parts, residual, gamma, eps, int64_sizes):

@@ -14,6 +14,12 @@
  *                            (the kernel at impl.h:316-340 rounds once; the test composition, which is
  *                             the judged one, rounds twice — this file follows the test)
  *                   fp64 sum of squares as in test/unit_test.cpp:204-210 is mode TDO_SUMSQ_F64
+ *                   mean    test/test_all_reduce_fusion.py:25 `x.float().pow(2).mean(-1)`: the arithmetic is in
+ *                            torch (third party, not in the reference tree; 2.10.0 in this image).  Its CPU
+ *                            kernel sums a contiguous row with 8-float vectors, four interleaved vector
+ *                            accumulators and a cascade every 16 steps; tdo_torch_row_sum restates that order
+ *                            (mode TDO_SUMSQ_TORCH) and tests/test_oracle.py pins it bit for bit against
+ *                            torch.sum / torch.mean over every row length the tests and benchmarks use.
  *   quant (PARITY UNPINNED by the reference, which has no quant code): scale = amax/qmax,
  *                   code = rne(clamp(y/scale)), OCP e4m3 (bias 7, no infinities, NaN = 0x7f) or int8.
  *
@@ -36,6 +42,7 @@
 #define TDO_SUMSQ_F32_SEQ 0  /* fp32 accumulator, left to right */
 #define TDO_SUMSQ_F64 1      /* fp64 accumulator, rounded to fp32 once (closest to the exact mean) */
 #define TDO_SUMSQ_F32_PAIRWISE 2 /* fp32 pairwise tree over the row */
+#define TDO_SUMSQ_TORCH 3    /* the order of torch's CPU sum over a contiguous row (tdo_torch_row_sum) */
 
 static uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
 static float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
@@ -163,6 +170,79 @@ static float round_elem(int dtype, float v) {
     }
 }
 
+/*
+ * Sum of n floats in the order torch's CPU kernel uses for a reduction over a contiguous row on x86
+ * (vector width 8 floats, four interleaved accumulators, partial sums flushed to the next cascade level
+ * every 2^level_power steps).  Rows shorter than one vector take four interleaved scalars instead.
+ */
+static int ceil_log2_i64(int64_t x) {
+    if (x <= 2) return 1;
+    int n = 0;
+    for (uint64_t v = (uint64_t)(x - 1); v; v >>= 1) ++n;
+    return n;
+}
+
+/* nrows interleaved accumulators of `width` floats each over `size` steps; step i, accumulator k reads
+   v[(i * nrows + k) * width + lane].  out[nrows][width]. */
+static void cascade_rows(const float *v, int64_t size, int nrows, int width, float *out) {
+    enum { LEVELS = 4 };
+    float acc[LEVELS][4][8];
+    memset(acc, 0, sizeof(acc));
+    int level_power = ceil_log2_i64(size) / LEVELS;
+    if (level_power < 4) level_power = 4;
+    const int64_t level_step = (int64_t)1 << level_power;
+    const int64_t level_mask = level_step - 1;
+    int64_t i = 0;
+    while (i + level_step <= size) {
+        for (int64_t j = 0; j < level_step; ++j, ++i)
+            for (int k = 0; k < nrows; ++k)
+                for (int l = 0; l < width; ++l) acc[0][k][l] += v[(i * nrows + k) * width + l];
+        for (int j = 1; j < LEVELS; ++j) {
+            for (int k = 0; k < nrows; ++k)
+                for (int l = 0; l < width; ++l) { acc[j][k][l] += acc[j - 1][k][l]; acc[j - 1][k][l] = 0.0f; }
+            const int64_t mask = level_mask << (j * level_power);
+            if ((i & mask) != 0) break;
+        }
+    }
+    for (; i < size; ++i)
+        for (int k = 0; k < nrows; ++k)
+            for (int l = 0; l < width; ++l) acc[0][k][l] += v[(i * nrows + k) * width + l];
+    for (int j = 1; j < LEVELS; ++j)
+        for (int k = 0; k < nrows; ++k)
+            for (int l = 0; l < width; ++l) acc[0][k][l] += acc[j][k][l];
+    for (int k = 0; k < nrows; ++k)
+        for (int l = 0; l < width; ++l) out[k * width + l] = acc[0][k][l];
+}
+
+/* One accumulator group of `width` lanes over `count` items of `width` floats: four interleaved partial sums,
+   the items left over added to the first, then the other three added to it. */
+static void row_sum_lanes(const float *v, int64_t count, int width, float *out) {
+    float part[4 * 8];
+    const int64_t size_ilp = count / 4;
+    cascade_rows(v, size_ilp, 4, width, part);
+    for (int64_t i = size_ilp * 4; i < count; ++i)
+        for (int l = 0; l < width; ++l) part[l] += v[i * width + l];
+    for (int k = 1; k < 4; ++k)
+        for (int l = 0; l < width; ++l) part[l] += part[k * width + l];
+    for (int l = 0; l < width; ++l) out[l] = part[l];
+}
+
+float tdo_torch_row_sum(const float *v, int64_t n) {
+    enum { W = 8 };
+    if (n < W) {
+        float s;
+        row_sum_lanes(v, n, 1, &s);
+        return s;
+    }
+    float lanes[W];
+    const int64_t vecs = n / W;
+    row_sum_lanes(v, vecs, W, lanes);
+    float s = 0.0f;
+    for (int64_t k = vecs * W; k < n; ++k) s += v[k];
+    for (int l = 0; l < W; ++l) s += lanes[l];
+    return s;
+}
+
 static float pairwise_sum(const float *v, int64_t n) {
     if (n <= 8) {
         float s = 0.0f;
@@ -207,6 +287,8 @@ int tdo_reduce_rms(int dtype, int nranks, int64_t tokens, int64_t hidden, const 
             sumsq = (float)d;
         } else if (sumsq_mode == TDO_SUMSQ_F32_PAIRWISE) {
             sumsq = pairwise_sum(sq, hidden);
+        } else if (sumsq_mode == TDO_SUMSQ_TORCH) {
+            sumsq = tdo_torch_row_sum(sq, hidden);
         } else {
             sumsq = 0.0f;
             for (int64_t h = 0; h < hidden; ++h) sumsq += sq[h];

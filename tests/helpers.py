@@ -38,12 +38,13 @@ def bits_equal(a: torch.Tensor, b: torch.Tensor) -> bool:
 
 
 def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, write_norm=None, use_table=False,
-            rank=0, device="cuda:0", static_scale=0.0, stage_init=None, calls=None):
+            rank=0, device="cuda:0", static_scale=0.0, stage_init=None, calls=None, vecs_per_thread=0, rows_per_block=0):
     """Run the HIP path through the C ABI (tde_reduce_rms) on CPU inputs; returns CPU outputs.
     parts: [N,T,H] tensor or list of N [T,H] tensors.  stage_init: [T,H] initial content of the stage
     buffer (staged algorithms); the stage is then returned as out["stage"].  calls: sequence of
     (phases, rank) issued in order on the same buffers instead of the one tde_reduce_rms call, e.g.
-    [(("reduce",), 0), (("reduce",), 1), (("norm",), 0)]."""
+    [(("reduce",), 0), (("reduce",), 1), (("norm",), 0)].  vecs_per_thread / rows_per_block: the per-call
+    launch-geometry overrides of tde_problem (0 = automatic)."""
     dev = torch.device(device)
     n = len(parts)
     T, H = residual.shape
@@ -83,7 +84,8 @@ def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, wri
     stream = torch.cuda.current_stream(dev).cuda_stream
     for phases, call_rank in (calls or [(("reduce", "norm"), rank)]):
         prob = _capi.make_problem(DTYPE_CODE[dtype], n, T, H, eps, quant=qm, algo=algo, write_norm=int(bool(write_norm)),
-                                  rank=call_rank, static_scale=static_scale)
+                                  rank=call_rank, static_scale=static_scale, vecs_per_thread=vecs_per_thread,
+                                  rows_per_block=rows_per_block)
         _capi.reduce_rms(prob, ptrs, d_res.data_ptr(), d_res_out.data_ptr(), d_gamma.data_ptr(),
                          norm_out=d_norm.data_ptr() if d_norm is not None else None,
                          q_out=d_q.data_ptr() if d_q is not None else None,
@@ -145,24 +147,19 @@ def quant_from_own_norm(norm_got, quant):
     return eager.quant_int8(norm_got)
 
 
-def check_against_oracle(got, want, quant, gamma=None, eps=None, norm_ulp=None, norm_flip_frac=2e-4, scale_rtol=1e-6,
-                         strict=False):
-    """Two levels.
+def check_against_oracle(got, want, quant, gamma=None, eps=None, strict=True):
+    """Every output bit for bit against the oracle's.
 
-    Stage-exact (needs gamma/eps and a norm_out from the kernel):
-      residual_out bit-exact; every normed row bit-identical to the eager composition for a reciprocal
-      RMS within 4 fp32 ulps of the oracle's; scales and codes bit-identical to the oracle's quantizer
-      applied to the kernel's own normed rows.
-    End to end against the oracle's outputs:
-      normed within 1 ulp except a fraction <= norm_flip_frac of elements (never more than norm_ulp):
-      those are elements whose first rounding lands on the other side because the reciprocal RMS
-      differs in its last fp32 bit; codes within one quant step; scales within scale_rtol relative,
-      except rows/groups whose maximum element is one of those flipped elements (counted, and bounded
-      by the number of flipped elements).
-    norm_ulp defaults to 2 (the second rounding can carry a first-rounding flip one step further); strict=True
-    (the bf16 benchmark configurations at the sizes the parity tests run them) demands 1 ulp (the stated bound:
-    normed bf16 within 1 bf16 ulp) and that no scale at all is outside scale_rtol.
-    Returns mismatch statistics."""
+    residual_out: fp32 rank-order sum, one rounding, residual add, one rounding (bit-exact by contract).
+    norm_out, scales, codes: bit-exact as well, because the kernel sums the squares in the order of torch's CPU
+    reduction (8-float vectors, four interleaved accumulators, a cascade every 16 steps: what every x86 host
+    with AVX2 or better runs, pinned in tests/test_oracle.py), divides and takes the square root in IEEE
+    arithmetic, and rounds twice like the eager composition.  The stated bounds (normed within 1 ulp, codes
+    within one quant step, scales within 1e-6 relative) are therefore met with zero differences.
+
+    strict=False relaxes norm_out/scales/codes to those stated bounds plus the allowance for a reciprocal RMS that
+    differs in its last bit (for a host whose torch sums in another order); the stage-exact checks stay.
+    Returns mismatch statistics (all zero when strict)."""
     stats = {}
     assert bits_equal(got["residual_out"], want["residual_out"]), "residual_out is not bit-exact"
     flipped = 0
@@ -174,34 +171,23 @@ def check_against_oracle(got, want, quant, gamma=None, eps=None, norm_ulp=None, 
         stats["norm_max_ulp"] = int(d.max()) if d.numel() else 0
         stats["norm_diff_elems"] = flipped
         stats["norm_gt1_elems"] = int((d > 1).sum())
-        if got["norm_out"].dtype == torch.float64:
-            # doubles scaled by an fp32 reciprocal RMS: a last-bit difference of that factor moves a whole row
-            # by 2^-24 relative.  End to end a relative bound; the stage-exact check below stays bit-exact.
-            rel = (got["norm_out"] - want["norm_out"]).abs() / want["norm_out"].abs().clamp_min(1e-300)
-            assert float(rel.max()) <= 4 * 2.0 ** -24
-            flipped = got["norm_out"].shape[0]
-        elif got["norm_out"].dtype == torch.float32:
-            # fp32 has no second rounding to absorb a last-bit difference of the reciprocal RMS: whole rows
-            # move by an ulp or two.  End to end the reference's own tolerance applies (atol 1e-4,
-            # test/unit_test.cpp:219); the stage-exact check below stays bit-exact.
-            assert stats["norm_max_ulp"] <= 8
-            magnitude = max(1.0, float(want["norm_out"].abs().max()))      # the reference's inputs are O(1)
-            assert float((got["norm_out"] - want["norm_out"]).abs().max()) <= 1e-4 * magnitude
-            flipped = got["norm_out"].shape[0]
-        else:
-            if norm_ulp is None:
-                norm_ulp = 1 if (strict and got["norm_out"].dtype == torch.bfloat16) else 2
-            assert stats["norm_max_ulp"] <= norm_ulp, (
-                "norm_out off by %d ulp (allowed %d: 1 for bf16; 2 for fp16, where a first rounding that lands on the "
-                "other side because the reciprocal RMS differs in its last fp32 bit can move the second rounding too)"
-                % (stats["norm_max_ulp"], norm_ulp))
-            assert flipped / n <= norm_flip_frac, "%d of %d normed elements differ" % (flipped, n)
         if gamma is not None:
             ok, matched = norm_rows_explained(got["norm_out"], got["residual_out"], gamma, eps)
             stats["rows_needing_rs_neighbour"] = int((matched > 0).sum())
             assert ok, "%d normed rows are not the eager composition for any reciprocal RMS within 4 ulps" % int(
                 (matched < 0).sum())
-    if quant != "none":
+        if strict:
+            assert bits_equal(got["norm_out"], want["norm_out"]), "norm_out differs in %d elements (max %d ulp)" % (
+                flipped, stats["norm_max_ulp"])
+        elif got["norm_out"].dtype in (torch.float32, torch.float64):
+            # no second rounding to absorb a last-bit difference of the reciprocal RMS: whole rows move by an ulp
+            # or two; the reference's own tolerance (atol 1e-4, test/unit_test.cpp:219) bounds it
+            magnitude = max(1.0, float(want["norm_out"].abs().max()))
+            assert float((got["norm_out"] - want["norm_out"]).abs().max()) <= 1e-4 * magnitude
+            flipped = got["norm_out"].shape[0]
+        else:
+            assert stats["norm_max_ulp"] <= 2 and flipped / n <= 2e-4
+    if quant != "none" and quant != "fp8_static":
         if "norm_out" in got:
             q_own, s_own = quant_from_own_norm(got["norm_out"], quant)
             assert bits_equal(got["scale"].reshape(-1), s_own.reshape(-1)), "scales differ from amax(own normed rows)/qmax"
@@ -210,21 +196,21 @@ def check_against_oracle(got, want, quant, gamma=None, eps=None, norm_ulp=None, 
         gs, ws = got["scale"].double().flatten(), want["scale"].double().flatten()
         rel = (gs - ws).abs() / ws.abs().clamp_min(1e-30)
         rel = torch.where((gs == 0) & (ws == 0), torch.zeros_like(rel), rel)
-        bad = int((rel > scale_rtol).sum())
         stats["scale_max_rel"] = float(rel.max()) if rel.numel() else 0.0
-        stats["scale_bad"] = bad
-        if strict:
-            assert bad == 0, "%d scales differ by more than %g relative (max %g)" % (bad, scale_rtol, stats["scale_max_rel"])
-        # otherwise (fp16/fp32 rows, randomized and extreme-magnitude cases): a scale may differ only where the row's
-        # maximum is one of the elements whose rounding flipped with the last bit of the reciprocal RMS
-        assert bad <= flipped, "%d scales differ by more than %g relative (max %g) with only %d flipped elements" % (
-            bad, scale_rtol, stats["scale_max_rel"], flipped)
-        assert stats["scale_max_rel"] <= 2.0 ** -7, "a scale is off by more than one ulp of the element type"
+        stats["scale_bad"] = int((rel > 1e-6).sum())
         if quant == "int8_token":
             dq = (got["q"].to(torch.int32) - want["q"].to(torch.int32)).abs()
         else:
             dq = ulp_distance(got["q"], want["q"])
         stats["q_max_step"] = int(dq.max()) if dq.numel() else 0
         stats["q_diff_elems"] = int((dq > 0).sum())
-        assert stats["q_max_step"] <= 1, "codes off by %d quant steps" % stats["q_max_step"]
+        if strict:
+            assert bits_equal(got["scale"].reshape(-1), want["scale"].reshape(-1)), "%d scales differ (max %g relative)" % (
+                int((gs != ws).sum()), stats["scale_max_rel"])
+            assert bits_equal(got["q"], want["q"]), "%d codes differ" % stats["q_diff_elems"]
+        else:
+            assert stats["scale_bad"] <= flipped and stats["scale_max_rel"] <= 2.0 ** -7
+            assert stats["q_max_step"] <= 1, "codes off by %d quant steps" % stats["q_max_step"]
+    elif quant == "fp8_static" and "q" in want:
+        assert bits_equal(got["q"], want["q"]), "static-scale codes differ"
     return stats

@@ -26,11 +26,11 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), name
     assert sorted(_capi.EXPORTS) == declared
-    assert _capi.load().tde_abi_version() == 1
+    assert _capi.load().tde_abi_version() == 2
 
 
 def test_struct_layouts_match_header():
-    assert ctypes.sizeof(_capi.Problem) == 48
+    assert ctypes.sizeof(_capi.Problem) == 56
     assert ctypes.sizeof(_capi.Buffers) == (16 + 8) * 8
     assert ctypes.sizeof(_capi.PlanOut) == 48
 
@@ -54,12 +54,34 @@ def _plan(**kw):
     (dict(quant=9), _capi.EQUANT), (dict(quant=_capi.QUANT_FP8_GROUP, hidden=1032), _capi.EQUANT),
     (dict(quant=_capi.QUANT_FP8_STATIC), _capi.EQUANT), (dict(quant=_capi.QUANT_FP8_STATIC, static_scale=-2.0), _capi.EQUANT),
     (dict(algo=5), _capi.EALGO), (dict(rank=8), _capi.ERANK), (dict(rank=-1), _capi.ERANK),
+    (dict(hidden=1 << 40), _capi.EHIDDEN),  # far beyond a row: refused before any size arithmetic
+    (dict(vecs_per_thread=3), _capi.EINVAL), (dict(rows_per_block=-1), _capi.EINVAL),   # per-call geometry overrides
 ])
 def test_plan_rejects(kw, status):
     with pytest.raises(_capi.TdeError) as e:
         _plan(**kw)
     assert e.value.status == status
     assert _capi.status_string(status) != "unknown status"
+
+
+def test_static_stage_entry_point_limits_need_no_gpu():
+    lib = _capi.load()
+    b = _capi.Buffers()
+    prob = _capi.make_problem(_capi.BF16, 8, 2049, 8192, 1e-6)       # one row more than the 32 MiB stage holds
+    assert lib.tde_reduce_rms_static_stage(ctypes.byref(prob), ctypes.byref(b), None) == _capi.ETOOBIG
+    for algo in (_capi.ALGO_FUSED, _capi.ALGO_STAGED_OWNED):
+        prob = _capi.make_problem(_capi.BF16, 8, 16, 1024, 1e-6, algo=algo)
+        assert lib.tde_reduce_rms_static_stage(ctypes.byref(prob), ctypes.byref(b), None) == _capi.EALGO
+    assert lib.tde_reduce_rms_static_stage(None, None, None) == _capi.EINVAL
+
+
+def test_plan_geometry_overrides_are_per_call():
+    auto = _plan()
+    forced = _plan(vecs_per_thread=1)
+    assert auto.vecs_per_thread == 4 and forced.vecs_per_thread == 1 and forced.block_threads == 1024
+    assert _plan().vecs_per_thread == 4          # nothing sticks between calls
+    packed = _plan(hidden=1024, tokens=4096, vecs_per_thread=1, rows_per_block=4)
+    assert packed.rows_per_block == 4 and packed.block_threads == 512 and packed.grid_blocks == 1024
 
 
 def test_plan_null_pointers():

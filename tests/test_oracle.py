@@ -155,6 +155,60 @@ def test_rmsnorm_torch_vs_c_restatement_and_fp64(dtype, code):
     assert rel < {torch.bfloat16: 2 ** -7, torch.float16: 2 ** -10, torch.float32: 2 ** -21}[dtype]
 
 
+@pytest.mark.parametrize("n", [2, 4, 6, 8, 9, 33, 64, 100, 124, 258, 508, 512, 1016, 1024, 2048, 3584, 4096, 5120, 7168, 8192])
+def test_sum_order_of_the_mean_of_squares_is_pinned(n):
+    """The eager composition's mean of squares (test/test_all_reduce_fusion.py:25) is computed by torch's CPU
+    reduction, whose summation order decides the last bit of the reciprocal RMS.  The C restatement of that
+    order (tdo_torch_row_sum) must give torch's sum, mean and rsqrt bit for bit, at every row length the tests
+    and benchmark configurations use and at one, many and odd numbers of rows (threads split rows, never a row)."""
+    g = torch.Generator().manual_seed(1000 + n)
+    for rows in (1, 7, 300):
+        x = (torch.randn(rows, n, generator=g) * 1.7).to(torch.bfloat16)
+        sq = x.float().pow(2)
+        got = cport.torch_row_sums(sq.numpy())
+        assert np.array_equal(got.view(np.uint32), sq.sum(-1).numpy().view(np.uint32)), (n, rows)
+        mean = got / np.float32(n)
+        assert np.array_equal(mean.view(np.uint32), sq.mean(-1).numpy().view(np.uint32))
+        rs = np.float32(1.0) / np.sqrt(mean + np.float32(1e-5), dtype=np.float32)
+        want = torch.rsqrt(sq.mean(-1) + 1e-5).numpy()
+        assert np.array_equal(rs.astype(np.float32).view(np.uint32), want.view(np.uint32))
+
+
+def test_sum_order_distinguishes_plausible_mistakes():
+    """A sequential, a pairwise and an fp64 sum all differ from torch's order on ordinary data: the pin above
+    cannot be met by a restatement that gets the order wrong."""
+    g = torch.Generator().manual_seed(7)
+    sq = torch.randn(400, 4096, generator=g).pow(2)
+    want = sq.sum(-1).numpy()
+    a = sq.numpy()
+    seq = np.zeros(400, dtype=np.float32)
+    for k in range(4096):
+        seq = seq + a[:, k]
+    f64 = a.astype(np.float64).sum(-1).astype(np.float32)
+    assert (seq != want).any() and (f64 != want).any()
+    assert np.array_equal(cport.torch_row_sums(a).view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("dtype,code", [(torch.bfloat16, cport.BF16), (torch.float16, cport.F16), (torch.float32, cport.F32)])
+@pytest.mark.parametrize("hidden", [1024, 5120, 508])
+def test_c_restatement_in_torch_sum_order_is_bit_identical_to_eager(dtype, code, hidden):
+    if hidden == 508 and dtype != torch.float32:
+        hidden = 504
+    p, r, g = eager.make_inputs(4, 29, hidden, dtype, 1.0, seed=hidden)
+    want = eager.reduce_rms(p, r, g, 1e-6, "fp8_token" if hidden % 8 == 0 else "none")
+    if dtype == torch.float32:
+        conv, back = (lambda t: t.numpy()), (lambda a: torch.from_numpy(a))
+    else:
+        conv, back = _bits16, (lambda a: _from_bits16(a, dtype))
+    quant = "fp8_token" if hidden % 8 == 0 else "none"
+    c = cport.reduce_rms(code, [conv(p[i]) for i in range(4)], conv(r), conv(g), 1e-6, quant=quant, sumsq_mode=cport.SUMSQ_TORCH)
+    assert bits_equal(back(c["residual_out"]), want["residual_out"])
+    assert bits_equal(back(c["norm_out"]), want["norm_out"])
+    if quant != "none":
+        assert np.array_equal(c["scale"].view(np.uint32), want["scale"].numpy().view(np.uint32))
+        assert np.array_equal(c["q"], want["q"].view(torch.uint8).numpy())
+
+
 def test_library_rms_norm_cross_check():
     p, r, g = eager.make_inputs(2, 8, 512, torch.bfloat16, 1.0, seed=9)
     x = eager.reduce_residual(p, r)

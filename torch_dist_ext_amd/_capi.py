@@ -20,7 +20,7 @@ ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, ALGO_STAGED_OWNED = 0, 1, 2, 3
 EXPORTS = (
     "tde_abi_version", "tde_status_string", "tde_last_hip_error", "tde_plan", "tde_reduce_rms", "tde_stage_reduce", "tde_stage_norm",
     "tde_reduce_rms_static_stage",
-    "tde_tune_override", "tde_probe_copy", "tde_probe_stream", "tde_probe_rows", "tde_device_info",
+    "tde_probe_copy", "tde_probe_stream", "tde_probe_rows", "tde_device_info",
     "tde_workspace_create", "tde_workspace_destroy", "tde_workspace_slot", "tde_workspace_stage",
     "tde_workspace_slot_bytes", "tde_workspace_nranks", "tde_workspace_fill_table",
 )
@@ -31,6 +31,7 @@ class Problem(ctypes.Structure):
         ("dtype", ctypes.c_int32), ("nranks", ctypes.c_int32), ("rank", ctypes.c_int32), ("quant", ctypes.c_int32),
         ("algo", ctypes.c_int32), ("write_norm", ctypes.c_int32), ("tokens", ctypes.c_int64), ("hidden", ctypes.c_int64),
         ("eps", ctypes.c_float), ("static_scale", ctypes.c_float),
+        ("tune_vecs_per_thread", ctypes.c_int32), ("tune_rows_per_block", ctypes.c_int32),
     ]
 
 
@@ -86,8 +87,6 @@ def load():
     for fn in (lib.tde_stage_reduce, lib.tde_stage_norm, lib.tde_probe_rows, lib.tde_reduce_rms_static_stage):
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(Problem), ctypes.POINTER(Buffers), ctypes.c_void_p]
-    lib.tde_tune_override.restype = ctypes.c_int
-    lib.tde_tune_override.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
     lib.tde_probe_copy.restype = ctypes.c_int
     lib.tde_probe_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
     lib.tde_probe_stream.restype = ctypes.c_int
@@ -125,9 +124,10 @@ def check(status):
 
 
 def make_problem(dtype, nranks, tokens, hidden, eps, quant=QUANT_NONE, algo=ALGO_AUTO, write_norm=0, rank=0,
-                 static_scale=0.0):
+                 static_scale=0.0, vecs_per_thread=0, rows_per_block=0):
     return Problem(dtype=dtype, nranks=nranks, rank=rank, quant=quant, algo=algo, write_norm=int(write_norm),
-                   tokens=tokens, hidden=hidden, eps=eps, static_scale=static_scale)
+                   tokens=tokens, hidden=hidden, eps=eps, static_scale=static_scale,
+                   tune_vecs_per_thread=vecs_per_thread, tune_rows_per_block=rows_per_block)
 
 
 def plan(problem):
@@ -154,10 +154,6 @@ def reduce_rms(problem, partials, residual_in, residual_out, gamma, norm_out=Non
           ("norm",): lib.tde_stage_norm, ("traffic",): lib.tde_probe_rows,
           ("static_stage",): lib.tde_reduce_rms_static_stage}[tuple(phases)]
     check(fn(ctypes.byref(problem), ctypes.byref(b), stream))
-
-
-def tune_override(vecs_per_thread=0, rows_per_block=0, max_grid=0):
-    check(load().tde_tune_override(vecs_per_thread, rows_per_block, max_grid))
 
 
 def device_info():

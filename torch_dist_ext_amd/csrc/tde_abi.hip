@@ -59,13 +59,28 @@ int static_stage_ptr(void **out) {
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 constexpr int kMaxBlock = 1024;
+constexpr int kDefaultComputeUnits = 256; // MI355X; used when no device can be asked (planning on a host without one)
 
-// Tuning override for sweeps (0 = automatic).
-int g_force_vpt = 0;
-int g_force_rows_per_block = 0;
-int g_force_grid = 0;
-
-constexpr int kComputeUnits = 256; // MI355X
+// Compute units of the current device, asked once per device.
+int compute_units() {
+    static std::mutex mu;
+    static int cached[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return kDefaultComputeUnits;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (cached[dev] == 0) {
+        int cu = 0;
+        if (hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cu <= 0) {
+            (void)hipGetLastError();
+            cu = kDefaultComputeUnits;
+        }
+        cached[dev] = cu;
+    }
+    return cached[dev];
+}
 
 int validate(const tde_problem *p, tde::Geometry *geo) {
     if (p == nullptr) return TDE_EINVAL;
@@ -74,6 +89,7 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     if (!(p->nranks == 2 || p->nranks == 4 || p->nranks == 8)) return TDE_ENRANKS;
     if (p->rank < 0 || p->rank >= p->nranks) return TDE_ERANK;
     if (p->tokens < 0 || p->hidden <= 0) return TDE_ESHAPE;
+    if (p->hidden > kMaxBlock * 16) return TDE_EHIDDEN; // also keeps hidden * eb far from overflow
     if ((p->hidden * eb) % 16 != 0) return TDE_ESHAPE;
     if (p->quant < TDE_QUANT_NONE || p->quant > TDE_QUANT_FP8_STATIC) return TDE_EQUANT;
     if (p->quant == TDE_QUANT_FP8_STATIC && !(p->static_scale > 0.0f && p->static_scale <= 3.0e38f)) return TDE_EQUANT;
@@ -102,18 +118,22 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     } else if ((nvec == 256 || (nvec == 512 && p->nranks >= 8)) && p->tokens >= 1024) {
         vpt = 4;
     }
-    if (g_force_vpt == 1 || g_force_vpt == 2 || g_force_vpt == 4) vpt = g_force_vpt;
+    if (p->tune_vecs_per_thread != 0) {
+        if (p->tune_vecs_per_thread != 1 && p->tune_vecs_per_thread != 2 && p->tune_vecs_per_thread != 4) return TDE_EINVAL;
+        vpt = p->tune_vecs_per_thread;
+    }
+    if (p->tune_rows_per_block < 0) return TDE_EINVAL;
     if (p->dtype == TDE_F64) vpt = 1;
     const int64_t lanes = (nvec + vpt - 1) / vpt;
     const int tpr = (int)((lanes + 63) / 64 * 64);
     int rpb = 256 / tpr; // pack short rows so a workgroup has at least four wavefronts
     if (rpb * tpr > kMaxBlock / vpt) rpb = (kMaxBlock / vpt) / tpr; // never beyond the kernel's launch bound
-    while (rpb > 1 && (p->tokens + rpb - 1) / rpb < 2 * kComputeUnits) rpb /= 2; // keep every CU busy first
+    const int cus = compute_units();
+    while (rpb > 1 && (p->tokens + rpb - 1) / rpb < 2 * cus) rpb /= 2; // keep every CU busy first
     if (rpb < 1) rpb = 1;
-    if (g_force_rows_per_block > 0 && g_force_rows_per_block * tpr <= kMaxBlock / vpt) rpb = g_force_rows_per_block;
+    if (p->tune_rows_per_block > 0 && p->tune_rows_per_block * tpr <= kMaxBlock / vpt) rpb = p->tune_rows_per_block;
     if (p->tokens > 0 && rpb > p->tokens) rpb = (int)p->tokens;
-    int64_t grid = (p->tokens + rpb - 1) / rpb;
-    if (g_force_grid > 0 && grid > g_force_grid) grid = g_force_grid;
+    const int64_t grid = (p->tokens + rpb - 1) / rpb; // one workgroup per group of rows, no loop
     if (grid > 0x7fffffff) return TDE_ESHAPE;
 
     if (geo) {
@@ -213,20 +233,13 @@ const char *tde_status_string(int status) {
 
 int tde_last_hip_error(void) { return g_last_hip_error; }
 
-int tde_tune_override(int32_t vecs_per_thread, int32_t rows_per_block, int32_t max_grid) {
-    g_force_vpt = vecs_per_thread;
-    g_force_rows_per_block = rows_per_block;
-    g_force_grid = max_grid;
-    return TDE_OK;
-}
-
 int tde_probe_copy(void *dst, const void *src, int64_t bytes, void *hip_stream) {
     if (dst == nullptr || src == nullptr || bytes < 0 || bytes % 16 != 0) return TDE_EINVAL;
     if (!aligned16(dst) || !aligned16(src)) return TDE_EALIGN;
     if (bytes == 0) return TDE_OK;
     const int64_t vecs = bytes / 16;
     int64_t blocks = (vecs + 255) / 256;
-    if (blocks > kComputeUnits * 16) blocks = kComputeUnits * 16;
+    if (blocks > compute_units() * 16) blocks = compute_units() * 16;
     hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(hip_stream), src, dst, vecs);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? TDE_OK : hip_fail(e);

@@ -30,10 +30,8 @@ __global__ void __launch_bounds__(1024 / VPT) traffic_kernel(const RowArgs a, ui
 #pragma unroll
     for (int j = 0; j < VPT; ++j) lane_off[j] = (uint32_t)(j * tpr + t) * 16u;
 
-    const int64_t row_stride = (int64_t)gridDim.x * a.rows_per_block;
-    for (int64_t row0 = (int64_t)xcd_chunked_block(blockIdx.x, gridDim.x, (uint32_t)a.xcd_chunk) * a.rows_per_block;
-         row0 < a.tokens; row0 += row_stride) {
-        const int64_t row = row0 + group;
+    {
+        const int64_t row = (int64_t)xcd_chunked_block(blockIdx.x, gridDim.x, (uint32_t)a.xcd_chunk) * a.rows_per_block + group;
         const uint32_t bytes = (row < a.tokens) ? row_bytes : 0u;
         const int64_t row_byte = row * (int64_t)row_bytes;
         RowLoads<NP, VPT> d;

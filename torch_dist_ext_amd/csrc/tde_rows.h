@@ -6,7 +6,8 @@
 // src/common/all_reduce_fusion_impl.h:280-298):
 //   s   = T( ((0 + p_0) + p_1) + ... + p_{N-1} )      fp32 accumulate in rank order, one rounding to T
 //   x   = T( float(s) + float(residual_in) )           -> residual_out            (impl.h:271-278)
-//   rs  = 1 / sqrt( sum(float(x)^2) / H + eps )        fp32, IEEE divide and sqrt
+//   rs  = 1 / sqrt( sum(float(x)^2) / H + eps )        fp32, IEEE divide and sqrt; the sum in the order of
+//                                                      torch's CPU reduction (sumsq_torch_order below)
 //   y1  = T( float(x) * rs )
 //   y   = T( float(gamma) * float(y1) )                -> norm_out
 //   per-token fp8 : scale = amax|y| / 448, code = e4m3( clamp(float(y)/scale, +-448) )
@@ -131,9 +132,6 @@ __device__ __forceinline__ float dpp_move(float v) {
         float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
 
-struct OpSum {
-    static __device__ __forceinline__ float f(float a, float b) { return a + b; }
-};
 struct OpMax {
     static __device__ __forceinline__ float f(float a, float b) { return fmaxf(a, b); }
 };
@@ -158,10 +156,8 @@ __device__ __forceinline__ float wave_reduce(float v) {
     return Op::f(Op::f(a, b), Op::f(c, d));
 }
 
-// Reduce over the `waves_per_row` wavefronts that share a row.  `slots` is this iteration's LDS
-// buffer indexed by wavefront number inside the block; the caller alternates between two buffers
-// so that one barrier per reduction is enough.  Identity is 0 for both operators as used here
-// (sums of squares and maxima of absolute values).
+// Reduce over the `waves_per_row` wavefronts that share a row.  `slots` is an LDS buffer indexed by wavefront
+// number inside the block, used once per kernel (one barrier).  Identity is 0 (maxima of absolute values).
 template <class Op>
 __device__ __forceinline__ float row_reduce(float v, float *slots, int wave, int lane, int first_wave,
                                             int waves_per_row) {
@@ -172,6 +168,172 @@ __device__ __forceinline__ float row_reduce(float v, float *slots, int wave, int
     const int k = lane & 15;
     const float t = (k < waves_per_row) ? slots[first_wave + k] : 0.0f;
     return row16_reduce<Op>(t);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Sum of a row's squares in the order of torch's CPU reduction.
+//
+// The eager composition computes x.float().pow(2).mean(-1) (test/test_all_reduce_fusion.py:25).  On x86 hosts
+// torch reduces a contiguous row of n floats with 8-lane vectors and four interleaved vector accumulators
+// (its cascade sum): with V = n / 8 vectors, I = V / 4,
+//   chain (m, k), m = 0..7, k = 0..3, takes the elements 8 * (4 * i + k) + m, i = 0..I-1;
+//   every 16 consecutive i form a block that is summed left to right from zero; the block sums of a chain are
+//   summed left to right (a last block shorter than 16 included);
+//   p[m] = chain(m,0) + the V % 4 vectors left over + chain(m,1) + chain(m,2) + chain(m,3), left to right;
+//   sum  = the n % 8 scalars left over, then p[0] .. p[7], left to right from zero.
+// (Rows shorter than 8 floats use four interleaved scalars instead; rows beyond 8192 floats would add a cascade
+// level and do not occur: a row has at most 1024 16-byte vectors.)  Following that order makes the reciprocal RMS,
+// and with it every normed element, scale and code, bit-identical to the eager composition's.
+//
+// The row's squares are laid out in LDS in element order (`img`); one thread sums one block of one chain
+// (16 reads 32 floats apart), the block sums go through LDS (`bs`), and lanes 4m+k of every wavefront finish chain
+// (m, k).  With 8 floats per 16-byte vector (2-byte element types) a block of 64 vectors is exactly what one
+// wavefront loaded with one load instruction, so the first step needs no workgroup barrier (WAVE_BLOCKS).
+// ---------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float quad_bcast(float v) {
+    return dpp_move<CTRL>(v);
+}
+
+// Dynamic LDS a kernel that calls sumsq_torch_order needs.
+inline size_t sumsq_lds_bytes(int block_threads, int vpt, int vec_floats) {
+    return ((size_t)block_threads * vpt * vec_floats + 1024) * sizeof(float);
+}
+
+// Returns `v`, but only once `after` exists: index arithmetic built on the result cannot be hoisted above the
+// row loads, whose registers leave no room for it.
+__device__ __forceinline__ int not_before(int v, uint32_t after) {
+    asm volatile("; index math stays behind the row loads" : "+v"(v) : "v"(after));
+    return v;
+}
+
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Block `b` of chain `cl` (= 4m + k): the first `terms` (0..16) of 16 elements 32 floats apart, summed left to
+// right.  GUARD: never read past the last term (rows whose LDS image ends inside the block).
+template <bool GUARD>
+__device__ __forceinline__ float chain_block_sum(const float *img, int b, int cl, int terms) {
+    const float *src = img + 512 * b + 8 * (cl & 3) + (cl >> 2);
+    float v[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = src[(!GUARD || i < terms) ? 32 * i : 0];
+    float acc = 0.0f;
+    if (__builtin_amdgcn_ballot_w64(terms != 16) == 0) { // every lane of the wavefront has a full block
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc += v[i];
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc += (i < terms) ? v[i] : 0.0f;
+    }
+    return acc;
+}
+
+// Wavefront-uniform variant of not_before (the value comes back in a scalar register).
+__device__ __forceinline__ int uniform_not_before(int v, uint32_t after) {
+    return __builtin_amdgcn_readfirstlane(not_before(v, after));
+}
+
+// The squares of this thread's vector j (vector index j * tpr + t of the row) go to their place in the row group's
+// image, which holds the row's squares in element order.  `after`: a word of the data the squares were computed from.
+template <int VPT, int VECF>
+__device__ __forceinline__ void sumsq_put(float *lds_img, int j, int tpr, int group, int t, const float (&sq)[VECF], uint32_t after) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const int vec = not_before(group * (tpr * VPT) + j * tpr + t, after);
+    float *dst = lds_img + vec * VECF;
+    if constexpr (VECF % 4 == 0) {
+#pragma unroll
+        for (int c = 0; c < VECF; c += 4) *reinterpret_cast<f32x4 *>(dst + c) = f32x4{sq[c], sq[c + 1], sq[c + 2], sq[c + 3]};
+    } else {
+#pragma unroll
+        for (int c = 0; c < VECF; ++c) dst[c] = sq[c];
+    }
+}
+
+// After every thread of the row group has put its squares: the sum, the same value in every thread.
+// lds_img: one float per element the workgroup holds (threads * VPT * VECF), lds_bs: 1024 floats (32 per block),
+// both shared by the workgroup's row groups (sumsq_lds_bytes gives the total).
+// Contains workgroup barriers when a row spans several wavefronts: all threads of the workgroup must call it together.
+template <int VPT, int VECF, bool WAVE_BLOCKS>
+__device__ __forceinline__ float sumsq_torch_order(float *lds_img, float *lds_bs, int n, int t, int tpr, int group, int lane,
+                                                   uint32_t after) {
+    n = uniform_not_before(n, after);
+    tpr = uniform_not_before(tpr, after);
+    group = uniform_not_before(group, after);
+    t = not_before(t, after);
+    lane = not_before(lane, after);
+    const int waves_per_row = tpr >> 6;
+    const int cap = tpr * VPT * VECF;        // floats this row group can hold
+    const int cap_blocks = (cap + 511) >> 9; // 64-vector blocks this row group can hold (<= 16)
+    float *img = lds_img + group * cap;
+    float *bs = lds_bs + group * (cap_blocks * 32);
+    const int V = n >> 3, tail = n & 7, I = V >> 2, L = V & 3, NB = (I + 15) >> 4;
+
+    const int cl = lane & 31;
+    int blocks = NB; // block sums that exist in `bs`
+    if constexpr (WAVE_BLOCKS) {
+        static_assert(VECF == 8, "one wavefront load = one block of 64 eight-float vectors");
+        // Block j * waves_per_row + w is what wavefront w wrote for its vector j: no other wavefront is involved.
+        // Blocks past the row's end sum to zero, and adding zero to a sum of squares changes nothing.
+        wave_lds_fence();
+        const int w = t >> 6;
+#pragma unroll
+        for (int s = 0; s < (VPT + 1) / 2; ++s) {
+            const int j = (lane >> 5) + 2 * s;
+            if (j < VPT) {
+                const int b = j * waves_per_row + w;
+                int terms = I - 16 * b;
+                terms = terms < 0 ? 0 : (terms > 16 ? 16 : terms);
+                bs[b * 32 + cl] = chain_block_sum<false>(img, b, cl, terms);
+            }
+        }
+        blocks = cap_blocks;
+    } else {
+        if (waves_per_row > 1) __syncthreads(); else wave_lds_fence();
+        for (int c = t; c < 32 * NB; c += tpr) {
+            const int b = c >> 5;
+            int terms = I - 16 * b;
+            terms = terms > 16 ? 16 : terms;
+            bs[c] = chain_block_sum<true>(img, b, c & 31, terms);
+        }
+    }
+    if (waves_per_row > 1) __syncthreads(); else wave_lds_fence();
+
+    // Lane 4m + k of every wavefront sums the blocks of chain (m, k); the quad then holds the four chains of m.
+    float v[16];
+#pragma unroll
+    for (int b2 = 0; b2 < 16; ++b2) v[b2] = bs[(b2 < blocks ? b2 : 0) * 32 + cl];
+    float chain = 0.0f;
+#pragma unroll
+    for (int b2 = 0; b2 < 16; ++b2) chain += (b2 < blocks) ? v[b2] : 0.0f;
+    const int m = cl >> 2;
+    float p = quad_bcast<0x00>(chain);
+    for (int l = 0; l < L; ++l) p += img[8 * (4 * I + l) + m];
+    p += quad_bcast<0x55>(chain);
+    p += quad_bcast<0xAA>(chain);
+    p += quad_bcast<0xFF>(chain);
+
+    float sum = 0.0f;
+    if (V == 0) {
+        // fewer than 8 floats: four interleaved scalars, the first of them also takes what is left over
+        if (n < 4) {
+            for (int e = 0; e < n; ++e) sum += img[e];
+        } else {
+            sum = img[0];
+            for (int e = 4; e < n; ++e) sum += img[e];
+            sum += img[1];
+            sum += img[2];
+            sum += img[3];
+        }
+    } else {
+        for (int e = 0; e < tail; ++e) sum += img[8 * V + e];
+    }
+#pragma unroll
+    for (int mm = 0; mm < 8; ++mm) sum += read_lane(p, 4 * mm);
+    return sum;
 }
 
 // Every buffer is device (global) memory: the few accesses that do not go through a buffer resource
@@ -284,16 +446,17 @@ __global__ void __launch_bounds__(1024 / VPT)
     // output at the end (one write burst per row: 0.9 % faster on 8 x [2048, 8192] bf16 -> fp8); with fewer
     // partials storing as soon as the sum is known measures 0.6-1.3 % faster.
     constexpr bool LATE_RESIDUAL = (N >= 8);
-    __shared__ float lds_sum[2][kMaxWavesPerBlock];
-    __shared__ float lds_max[2][kMaxWavesPerBlock];
+    // Dynamic LDS: the workgroup's squares (one float per element it holds), then 1024 floats of block sums.
+    extern __shared__ __attribute__((aligned(16))) float lds_dyn[];
+    float *const lds_img = lds_dyn;
+    float *const lds_bs = lds_dyn + blockDim.x * (VPT * VEC);
+    __shared__ float lds_max[kMaxWavesPerBlock];
 
     const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int tpr = a.threads_per_row;
     const int waves_per_row = tpr >> 6;
     const int group = __builtin_amdgcn_readfirstlane(tid / tpr); // uniform inside a wavefront
-    const int t = tid - group * tpr;
     const int first_wave = group * waves_per_row;
     const uint32_t row_bytes = (uint32_t)a.hidden * E::BYTES;
 
@@ -312,7 +475,11 @@ __global__ void __launch_bounds__(1024 / VPT)
 
     uint32_t lane_off[VPT]; // byte offset of this thread's vector j inside a row
 #pragma unroll
-    for (int j = 0; j < VPT; ++j) lane_off[j] = (uint32_t)(j * tpr + t) * 16u;
+    for (int j = 0; j < VPT; ++j) lane_off[j] = (uint32_t)(j * tpr + tid - group * tpr) * 16u;
+// Thread index inside the row group and lane index, rebuilt from the first load offset where they are needed:
+// the thread id itself does not stay in a register through the load phase, which has none to spare.
+#define TDE_T ((int)(lane_off[0] >> 4))
+#define TDE_LANE ((int)(lane_off[0] >> 4) & (kWave - 1))
 
     auto issue_loads = [&](RowLoads<NP, VPT> &d, int64_t row) {
         const uint32_t bytes = (row < a.tokens) ? row_bytes : 0u;
@@ -328,10 +495,11 @@ __global__ void __launch_bounds__(1024 / VPT)
         for (int j = 0; j < VPT; ++j) d.r[j] = rsrc_load16(rr, lane_off[j]);
     };
 
-    const int64_t row_stride = (int64_t)gridDim.x * a.rows_per_block;
-    int64_t row0 = (int64_t)xcd_chunked_block(blockIdx.x, gridDim.x, (uint32_t)a.xcd_chunk) * a.rows_per_block;
+    // One workgroup, one group of rows: the grid covers every row (no loop; a looping wavefront waits for its
+    // own stores, a fresh workgroup does not).
+    const int64_t row0 = (int64_t)xcd_chunked_block(blockIdx.x, gridDim.x, (uint32_t)a.xcd_chunk) * a.rows_per_block;
 
-    // The first row's loads go out before anything else touches memory.
+    // The row's loads go out before anything else touches memory.
     RowLoads<NP, VPT> cur;
     issue_loads(cur, row0 + group);
     const rsrc_t gamma_rsrc = row_rsrc(a.gamma, 0, row_bytes);
@@ -341,8 +509,7 @@ __global__ void __launch_bounds__(1024 / VPT)
         gamma_early = __builtin_amdgcn_raw_buffer_load_b128(gamma_rsrc, (int)lane_off[0], 0, kAuxDefault);
     }
 
-    int parity = 0;
-    for (; row0 < a.tokens; row0 += row_stride, parity ^= 1) {
+    {
         const int64_t row = row0 + group;
         const bool row_ok = row < a.tokens;
         const uint32_t bytes = row_ok ? row_bytes : 0u;
@@ -351,7 +518,6 @@ __global__ void __launch_bounds__(1024 / VPT)
         // ---- reduce, residual add, sum of squares ------------------------------------------------
         const rsrc_t res_out = row_rsrc(a.residual_out, row_byte, bytes);
         u32x4 xraw[VPT];
-        float sumsq = 0.0f;
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
             float s[VEC];
@@ -377,12 +543,10 @@ __global__ void __launch_bounds__(1024 / VPT)
             xraw[j] = E::pack(x);
             if constexpr (!LATE_RESIDUAL) rsrc_store16(res_out, lane_off[j], xraw[j]);
             E::unpack(xraw[j], x);
+            float sq[VEC];
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                // 2-byte types: x*x is exact in fp32, so the fused form rounds exactly like mul-then-add.
-                if constexpr (E::BYTES == 2) sumsq = __builtin_fmaf(x[i], x[i], sumsq);
-                else sumsq += x[i] * x[i];
-            }
+            for (int i = 0; i < VEC; ++i) sq[i] = x[i] * x[i];
+            sumsq_put<VPT, VEC>(lds_img, j, tpr, group, TDE_T, sq, xraw[j][0]);
         }
         // gamma (shared by all rows, served from L2).  With several vectors per thread it is requested
         // only now: the registers of the row loads are free again, and the reduction below covers its
@@ -397,7 +561,7 @@ __global__ void __launch_bounds__(1024 / VPT)
         } else {
             gamma_raw[0] = gamma_early;
         }
-        sumsq = row_reduce<OpSum>(sumsq, lds_sum[parity], wave, lane, first_wave, waves_per_row);
+        const float sumsq = sumsq_torch_order<VPT, VEC, E::BYTES == 2>(lds_img, lds_bs, a.hidden, TDE_T, tpr, group, TDE_LANE, xraw[VPT - 1][0]);
         const float rs = 1.0f / __builtin_sqrtf(sumsq / a.hidden_f + a.eps);
 
         // ---- normalize ------------------------------------------------------------------------------
@@ -445,7 +609,7 @@ __global__ void __launch_bounds__(1024 / VPT)
                     float m = row16_reduce<OpMax>(amax[j]);
                     if constexpr (LANES_PER_GROUP == 32) m = fmaxf(m, __shfl_xor(m, 16, kWave));
                     scale[j] = m / QMAX;
-                    if ((lane & (LANES_PER_GROUP - 1)) == 0)
+                    if ((TDE_LANE & (LANES_PER_GROUP - 1)) == 0)
                         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, scale[j]), sc_out,
                                                               (int)((lane_off[j] / 16u / LANES_PER_GROUP) * 4u), 0, kAuxDefault);
                 }
@@ -456,11 +620,11 @@ __global__ void __launch_bounds__(1024 / VPT)
                 float m = amax[0];
 #pragma unroll
                 for (int j = 1; j < VPT; ++j) m = fmaxf(m, amax[j]);
-                m = row_reduce<OpMax>(m, lds_max[parity], wave, lane, first_wave, waves_per_row);
+                m = row_reduce<OpMax>(m, lds_max, wave, TDE_LANE, first_wave, waves_per_row);
                 const float sc = m / QMAX;
 #pragma unroll
                 for (int j = 0; j < VPT; ++j) scale[j] = sc;
-                if (row_ok && t == 0) ((TDE_GLOBAL float *)a.scale_out)[row] = sc;
+                if (row_ok && TDE_T == 0) ((TDE_GLOBAL float *)a.scale_out)[row] = sc;
             }
             const rsrc_t q_out = row_rsrc(a.q_out, row * (int64_t)a.hidden, row_ok ? (uint32_t)a.hidden : 0u);
             if constexpr (LATE_RESIDUAL) {
@@ -496,10 +660,10 @@ __global__ void __launch_bounds__(1024 / VPT)
                 }
             }
         }
-        // Only a capped grid comes round again; the next row's loads go out behind this row's stores.
-        if (row0 + row_stride < a.tokens) issue_loads(cur, row + row_stride);
     }
 }
+#undef TDE_T
+#undef TDE_LANE
 
 // Stage A of the staged algorithm: s = T(sum of partials) for every element, no row structure.
 // One workgroup of 256 threads reduces a contiguous span of 256*U vectors (U vectors per thread,
@@ -596,8 +760,9 @@ hipError_t launch_traffic(int n, int vpt, int code_bytes, bool wn, const RowArgs
 template <class E, int N, int VPT>
 hipError_t launch_rows_nv(int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s) {
     const dim3 grid((unsigned)g.grid), block((unsigned)g.block_threads);
-#define TDE_LAUNCH(QM, WNB)                                                       \
-    hipLaunchKernelGGL((row_kernel<E, N, VPT, QM, WNB>), grid, block, 0, s, a); \
+    const size_t lds = sumsq_lds_bytes(g.block_threads, VPT, E::VEC);
+#define TDE_LAUNCH(QM, WNB)                                                         \
+    hipLaunchKernelGGL((row_kernel<E, N, VPT, QM, WNB>), grid, block, lds, s, a); \
     return hipGetLastError();
     switch (q) {
     case TDE_QUANT_NONE: TDE_LAUNCH(TDE_QUANT_NONE, true)

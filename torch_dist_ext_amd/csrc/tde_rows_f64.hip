@@ -33,15 +33,14 @@ __device__ __forceinline__ u32x4 pack_f64(const double (&d)[2]) {
 
 template <int N>
 __global__ void __launch_bounds__(1024) row_kernel_f64(const RowArgs a) {
-    __shared__ float lds_sum[2][kMaxWavesPerBlock];
+    extern __shared__ __attribute__((aligned(16))) float lds_dyn[]; // squares (two per thread), then block sums
+    float *const lds_img = lds_dyn;
+    float *const lds_bs = lds_dyn + blockDim.x * 2;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
-    const int wave = tid >> 6;
     const int tpr = a.threads_per_row;
-    const int waves_per_row = tpr >> 6;
     const int group = __builtin_amdgcn_readfirstlane(tid / tpr);
     const int t = tid - group * tpr;
-    const int first_wave = group * waves_per_row;
     const uint32_t row_bytes = (uint32_t)a.hidden * 8u;
     const uint32_t off = (uint32_t)t * 16u;
 
@@ -57,10 +56,9 @@ __global__ void __launch_bounds__(1024) row_kernel_f64(const RowArgs a) {
     }
     const rsrc_t gamma_rsrc = row_rsrc(a.gamma, 0, row_bytes);
 
-    const int64_t row_stride = (int64_t)gridDim.x * a.rows_per_block;
-    int parity = 0;
-    for (int64_t row0 = (int64_t)blockIdx.x * a.rows_per_block; row0 < a.tokens; row0 += row_stride, parity ^= 1) {
-        const int64_t row = row0 + group;
+    {
+        const int64_t row = (int64_t)blockIdx.x * a.rows_per_block + group; // the grid covers every row
+
         const uint32_t bytes = (row < a.tokens) ? row_bytes : 0u;
         const int64_t row_byte = row * (int64_t)row_bytes;
         u32x4 praw[N];
@@ -84,9 +82,10 @@ __global__ void __launch_bounds__(1024) row_kernel_f64(const RowArgs a) {
         rsrc_store16(row_rsrc(a.residual_out, row_byte, bytes), off, pack_f64(x));
 
         const float f0 = (float)x[0], f1 = (float)x[1];
-        float sumsq = f0 * f0;
-        sumsq += f1 * f1;
-        sumsq = row_reduce<OpSum>(sumsq, lds_sum[parity], wave, lane, first_wave, waves_per_row);
+        const float sq[2] = {f0 * f0, f1 * f1};
+        const uint32_t landed = __builtin_bit_cast(uint32_t, sq[0]);
+        sumsq_put<1, 2>(lds_img, 0, tpr, group, t, sq, landed);
+        const float sumsq = sumsq_torch_order<1, 2, false>(lds_img, lds_bs, a.hidden, t, tpr, group, lane, landed);
         const float rs = 1.0f / __builtin_sqrtf(sumsq / a.hidden_f + a.eps);
 
         double g[2], y[2];
@@ -99,10 +98,11 @@ __global__ void __launch_bounds__(1024) row_kernel_f64(const RowArgs a) {
 
 hipError_t launch_rows_f64(int n, const RowArgs &a, const Geometry &g, hipStream_t s) {
     const dim3 grid((unsigned)g.grid), block((unsigned)g.block_threads);
+    const size_t lds = sumsq_lds_bytes(g.block_threads, 1, 2);
     switch (n) {
-    case 2: hipLaunchKernelGGL((row_kernel_f64<2>), grid, block, 0, s, a); break;
-    case 4: hipLaunchKernelGGL((row_kernel_f64<4>), grid, block, 0, s, a); break;
-    case 8: hipLaunchKernelGGL((row_kernel_f64<8>), grid, block, 0, s, a); break;
+    case 2: hipLaunchKernelGGL((row_kernel_f64<2>), grid, block, lds, s, a); break;
+    case 4: hipLaunchKernelGGL((row_kernel_f64<4>), grid, block, lds, s, a); break;
+    case 8: hipLaunchKernelGGL((row_kernel_f64<8>), grid, block, lds, s, a); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
