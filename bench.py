@@ -5,11 +5,15 @@ at 2048 x 8192 bf16 (the headline configuration, here called c3) on ONE MI355X, 
 A step is one launch of the fused row kernel over one batch of synthetic inputs that already sit
 in HBM.  Inputs and outputs rotate over enough distinct sets (> 4 GiB of inputs, > 1 GiB of
 outputs) that the 256 MB memory-side cache neither serves a launch's reads nor absorbs its writes.
+The first set is drawn on the CPU from the configuration's seed (the same tensors the parity tests use); the
+CPU-baseline leg runs the oracle on it and compares the kernel's outputs for that set bit for bit.
 Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3] [--no-cpu-baseline]
 """
 import argparse
+import ctypes
+import hashlib
 import json
 import os
 import sys
@@ -20,49 +24,88 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 
-# HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs summarized under
-# profiles/ (scaled by the plain-copy calibration described there); None where not collected.
-TRAFFIC_BYTES = {"c2": 11655354, "c3": 352644601, "c4": 765430448, "c5": 2182061403}
+# HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs summarized under profiles/
+# (scaled by the plain-copy calibration described there).  They describe the kernels whose sources hash to
+# `sources_sha256`; with any other kernel source the bench line reports traffic as null.
+TRAFFIC = {
+    "sources_sha256": "unmeasured",
+    "bytes": {},
+}
 
 BENCH_CONFIGS = {
-    # name: (N, T, H, dtype, sigma, eps, quant)
-    "c2": (8, 128, 4096, "bf16", 0.5, 1e-5, "none"),
-    "c3": (8, 2048, 8192, "bf16", 0.5, 1e-5, "fp8_token"),
-    "c4": (4, 8192, 7168, "bf16", 1.0, 1e-6, "fp8_group"),
-    "c5": (4, 32768, 5120, "f16", 1.0, 1e-6, "int8_token"),
+    # name: (N, T, H, dtype, sigma, eps, quant, seed, outlier_channels)
+    "c2": (8, 128, 4096, "bf16", 0.5, 1e-5, "none", 2, 0),
+    "c3": (8, 2048, 8192, "bf16", 0.5, 1e-5, "fp8_token", 3, 0),
+    "c4": (4, 8192, 7168, "bf16", 1.0, 1e-6, "fp8_group", 4, 0),
+    "c5": (4, 32768, 5120, "f16", 1.0, 1e-6, "int8_token", 5, 5),
 }
 
 
-def make_sets(torch, cfg, nsets, dev):
-    N, T, H, dt, sigma, eps, quant = cfg
+def kernel_sources_sha256():
+    """One hash over the kernel sources, so that figures measured with other kernels are not reported for these."""
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "torch_dist_ext_amd", "csrc")
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".h")):
+            with open(os.path.join(csrc, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()
+
+
+def seeded_cpu_inputs(torch, cfg):
+    """The configuration's inputs drawn on the CPU from its seed: partials ~ N(0, sigma), residual ~ N(0, 1),
+    gamma ~ U(0.5, 1.5), an optional fixed seeded set of outlier channels multiplied by 100 in every partial."""
+    N, T, H, dt, sigma, eps, quant, seed, outliers = cfg
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dt]
+    g = torch.Generator().manual_seed(seed)
+    parts = torch.randn((N, T, H), generator=g, dtype=torch.float32) * sigma
+    if outliers:
+        cols = torch.randperm(H, generator=g)[:outliers]
+        parts[:, :, cols] *= 100.0
+    residual = torch.randn((T, H), generator=g, dtype=torch.float32)
+    gamma = torch.rand((H,), generator=g, dtype=torch.float32) + 0.5
+    return parts.to(dtype), residual.to(dtype), gamma.to(dtype)
+
+
+def make_sets(torch, cfg, nsets, dev, first):
+    N, T, H, dt, sigma, eps, quant, seed, outliers = cfg
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dt]
     g = torch.Generator(device=dev).manual_seed(1234)
     sets = []
-    for _ in range(nsets):
-        parts = [(torch.randn((T, H), generator=g, device=dev, dtype=torch.float32) * sigma).to(dtype) for _ in range(N)]
-        residual = torch.randn((T, H), generator=g, device=dev, dtype=torch.float32).to(dtype)
+    for k in range(nsets):
+        if k == 0:
+            parts = [first[0][r].to(dev) for r in range(N)]
+            residual = first[1].to(dev)
+        else:
+            parts = [(torch.randn((T, H), generator=g, device=dev, dtype=torch.float32) * sigma).to(dtype) for _ in range(N)]
+            residual = torch.randn((T, H), generator=g, device=dev, dtype=torch.float32).to(dtype)
         res_out = torch.empty_like(residual)
         q = torch.empty((T, H), dtype=torch.uint8, device=dev) if quant != "none" else None
         nscale = T * (H // 128) if quant == "fp8_group" else T
         scale = torch.empty((nscale,), dtype=torch.float32, device=dev) if quant != "none" else None
         norm = torch.empty_like(residual) if quant == "none" else None
         sets.append(dict(parts=parts, residual=residual, res_out=res_out, q=q, scale=scale, norm=norm))
-    gamma = (torch.rand((H,), generator=g, device=dev, dtype=torch.float32) + 0.5).to(dtype)
-    return sets, gamma, dtype
+    return sets, first[2].to(dev), dtype
 
 
-def cpu_baseline(torch, cfg, budget_s=15.0):
-    """The oracle's torch-eager composition timed on the host cores, on a bounded sample: as many
-    full-size passes of the same workload as fit in about budget_s (at least 2 after one warm-up)."""
+def cpu_baseline(torch, cfg, first, kernel_out, budget_s=15.0):
+    """The oracle's torch-eager composition timed on the host cores, on a bounded sample: as many full-size
+    passes over the configuration's seeded inputs (at most 2048 rows of them) as fit in about budget_s (at least
+    2 after one warm-up).  The warm-up pass doubles as the checker of the kernel's outputs for the same rows."""
     from oracle import eager
-    N, T, H, dt, sigma, eps, quant = cfg
-    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dt]
+    N, T, H, dt, sigma, eps, quant, seed, outliers = cfg
     cores = os.cpu_count() or 1
-    cores = min(cores, 16)
-    torch.set_num_threads(cores)
+    threads = min(cores, 16)
+    torch.set_num_threads(threads)
     rows = min(T, 2048)
-    parts, residual, gamma = eager.make_inputs(N, rows, H, dtype, sigma, seed=3)
-    eager.reduce_rms(parts, residual, gamma, eps, quant)  # warm-up
+    parts, residual, gamma = first[0][:, :rows].contiguous(), first[1][:rows].contiguous(), first[2]
+    want = eager.reduce_rms(parts, residual, gamma, eps, quant)  # warm-up, and the expected outputs
+    checked = {}
+    for key, got in kernel_out.items():
+        ref = want[key].reshape(rows, -1)
+        g = got.reshape(T, -1)[:rows]
+        same = bool(torch.equal(g.contiguous().view(torch.uint8), ref.contiguous().view(torch.uint8)))
+        checked[key] = same
     times = []
     t_begin = time.perf_counter()
     while len(times) < 2 or (time.perf_counter() - t_begin < budget_s and len(times) < 50):
@@ -72,10 +115,11 @@ def cpu_baseline(torch, cfg, budget_s=15.0):
     times.sort()
     med = times[len(times) // 2]
     return {
-        "value": rows / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+        "value": rows / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "host_cpu_count": cores, "kind": "port",
         "sample": "%d passes of %d rows x %d (%s, N=%d, %s), median; torch-eager oracle on host CPU" % (
             len(times), rows, H, dt, N, quant),
         "ms_per_pass": med * 1e3,
+        "kernel_outputs_bit_identical_to_oracle": checked,
     }
 
 
@@ -88,7 +132,11 @@ def main():
     ap.add_argument("--sets", type=int, default=0, help="distinct input sets to rotate over (0 = enough for > 1 GiB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--algo", default="auto", choices=["auto", "fused", "staged", "staged_owned"])
+    ap.add_argument("--print-source-hash", action="store_true", help="print the kernel-source hash and exit")
     args = ap.parse_args()
+    if args.print_source_hash:
+        print(kernel_sources_sha256())
+        return
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (one rank's stage with N local partial buffers); "
               "--gpus %d with WORLD_SIZE=%s is not supported" % (args.gpus, os.environ.get("WORLD_SIZE", "1")), file=sys.stderr)
@@ -103,7 +151,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     cfg = BENCH_CONFIGS[args.config]
-    N, T, H, dt, sigma, eps, quant = cfg
+    N, T, H, dt, sigma, eps, quant, seed, outliers = cfg
     qm = {"none": _capi.QUANT_NONE, "fp8_token": _capi.QUANT_FP8_TOKEN, "fp8_group": _capi.QUANT_FP8_GROUP,
           "int8_token": _capi.QUANT_INT8_TOKEN}[quant]
     algo = {"auto": _capi.ALGO_AUTO, "fused": _capi.ALGO_FUSED, "staged": _capi.ALGO_STAGED,
@@ -118,7 +166,8 @@ def main():
     e = 2 if dt != "f32" else 4
     out_bytes = bytes_per_launch - (N + 1) * T * H * e - H * e
     nsets = args.sets or min(128, max(3, -(-(4 << 30) // bytes_per_launch), -(-(1 << 30) // max(out_bytes, 1))) + 1)
-    sets, gamma, dtype = make_sets(torch, cfg, nsets, dev)
+    first = seeded_cpu_inputs(torch, cfg)
+    sets, gamma, dtype = make_sets(torch, cfg, nsets, dev, first)
     staged = algo in (_capi.ALGO_STAGED, _capi.ALGO_STAGED_OWNED)
     # One stage buffer per input set, so that stage B reads it from HBM like everything else.
     stages = [torch.zeros((T, H), dtype=dtype, device=dev) for _ in range(nsets)] if staged else None
@@ -132,7 +181,6 @@ def main():
     stream = torch.cuda.current_stream(dev)
 
     # Argument blocks are built once per input set; a step is then a single C-ABI call.
-    import ctypes
     lib = _capi.load()
     calls = []
     for s in sets:
@@ -148,6 +196,20 @@ def main():
     prob_ref = ctypes.byref(prob)
     call_refs = [ctypes.byref(b) for b in calls]
     hip_stream = ctypes.c_void_p(stream.cuda_stream)
+
+    def timed(fn, steps, warmup):
+        """Average duration of `steps` back-to-back calls of fn(i) on the launch stream, by HIP events."""
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize(dev)
+        ev0 = torch.cuda.Event(enable_timing=True)
+        ev1 = torch.cuda.Event(enable_timing=True)
+        ev0.record(stream)
+        for i in range(steps):
+            fn(i)
+        ev1.record(stream)
+        torch.cuda.synchronize(dev)
+        return ev0.elapsed_time(ev1) * 1e3 / steps
 
     def launch(i):
         st = lib.tde_reduce_rms(prob_ref, call_refs[i % nsets], hip_stream)
@@ -183,35 +245,49 @@ def main():
     wall = time.perf_counter() - t0
     avg_ms = ev0.elapsed_time(ev1) / args.steps
 
-    # The same launches with the arithmetic removed (tde_probe_rows): what the access pattern alone takes
-    # on this box, in this process, over the same buffers.  It overwrites the outputs, hence after the timed run.
-    floor_us = None
+    # The kernel's outputs for the seeded set, kept for the checker in the CPU-baseline leg (the probes below
+    # overwrite the device copies).  Every timed launch of that set wrote the same values.
+    launch(0)
+    torch.cuda.synchronize(dev)
+    s0 = sets[0]
+    kernel_out = {"residual_out": s0["res_out"].cpu()}
+    if s0["norm"] is not None:
+        kernel_out["norm_out"] = s0["norm"].cpu()
+    if s0["q"] is not None:
+        kernel_out["q"] = s0["q"].cpu()
+        kernel_out["scale"] = s0["scale"].cpu()
+
+    # The same launches with the arithmetic removed (tde_probe_rows_parts): what the access pattern alone takes
+    # on this box, in this process, over the same buffers -- all of it, its input streams alone, its output
+    # streams alone.  They overwrite the outputs, hence after the timed run.
+    pattern = {}
     if not staged:
-        def launch_floor(i):
-            st = lib.tde_probe_rows(prob_ref, call_refs[i % nsets], hip_stream)
-            if st != 0:
-                _capi.check(st)
-        for i in range(args.warmup):
-            launch_floor(i)
-        torch.cuda.synchronize(dev)
-        ev2 = torch.cuda.Event(enable_timing=True)
-        ev3 = torch.cuda.Event(enable_timing=True)
-        ev2.record(stream)
-        for i in range(args.steps):
-            launch_floor(i)
-        ev3.record(stream)
-        torch.cuda.synchronize(dev)
-        floor_us = ev2.elapsed_time(ev3) * 1e3 / args.steps
+        for key, parts in (("traffic_only_us", 7), ("reads_only_us", 1), ("writes_only_us", 6)):
+            if parts == 6 and out_bytes <= 0:
+                continue
+
+            def launch_parts(i, parts=parts):
+                st = lib.tde_probe_rows_parts(prob_ref, call_refs[i % nsets], parts, hip_stream)
+                if st != 0:
+                    _capi.check(st)
+            pattern[key] = timed(launch_parts, args.steps, args.warmup)
+    floor_us = pattern.get("traffic_only_us")
+    read_bytes = (N + 1) * T * H * e
+    launch_floor_us = timed(lambda i: lib.tde_probe_launch(hip_stream), 500, 50)
 
     ms_per_step = wall * 1e3 / args.steps
     gbs_job = bytes_per_launch / (wall / args.steps) / 1e9
     achieved = bytes_per_launch / (avg_ms * 1e-3) / 1e9
+    traffic = None
+    if not staged and TRAFFIC["sources_sha256"] == kernel_sources_sha256():
+        traffic = TRAFFIC["bytes"].get(args.config)
     out = {
         "metric": ("achieved HBM GB/s, one rank's 8-partial reduce+residual+RMSNorm+per-token fp8 stage" if args.config == "c3"
                    else "achieved HBM GB/s, one rank's %d-partial reduce+residual+RMSNorm stage, quant=%s" % (N, quant)),
         "value": gbs_job, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",   # arithmetic is fp32 throughout; storage types are in config
+        # dtype is the arithmetic type (fp32 accumulate, norm and quant); tensors are stored as storage_dtype
+        "dtype": "f32", "storage_dtype": dt, "data": "synthetic",
         "tokens_per_s": T / (wall / args.steps),
         "pct_of_hbm_peak": 100.0 * gbs_job / HBM_PEAK_GBS,
         "config": {"workload": "%s: N=%d partials [%d,%d] %s, residual add + RMSNorm + %s%s" % (
@@ -221,11 +297,18 @@ def main():
                    "storage_dtype": dt, "output": quant, "algo": args.algo, "input_sets": nsets, "block_threads": plan.block_threads,
                    "grid_blocks": plan.grid_blocks, "algorithmic_bytes": bytes_per_launch},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None if staged else TRAFFIC_BYTES.get(args.config),
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel_avg_us": avg_ms * 1e3,
                      # the same launches without arithmetic (same bytes, same access pattern), and their share of the peak
                      "traffic_only_us": floor_us,
-                     "traffic_only_frac": (bytes_per_launch / (floor_us * 1e-6) / 1e9 / HBM_PEAK_GBS) if floor_us else None},
+                     "traffic_only_frac": (bytes_per_launch / (floor_us * 1e-6) / 1e9 / HBM_PEAK_GBS) if floor_us else None,
+                     # the pattern's input streams alone and output streams alone (same workgroups, no arithmetic)
+                     "reads_only_us": pattern.get("reads_only_us"),
+                     "reads_only_GBs": (read_bytes / (pattern["reads_only_us"] * 1e-6) / 1e9) if pattern.get("reads_only_us") else None,
+                     "writes_only_us": pattern.get("writes_only_us"),
+                     "writes_only_GBs": (out_bytes / (pattern["writes_only_us"] * 1e-6) / 1e9) if pattern.get("writes_only_us") else None,
+                     # one empty dispatch, back to back on the same stream: the floor under latency-bound sizes
+                     "launch_floor_us": launch_floor_us},
     }
     # The device's practical streaming rates, measured now (tde_probe_stream: 1 GiB per launch, four buffers
     # in rotation): what reads alone, writes alone and a plain copy reach on this box.
@@ -235,17 +318,9 @@ def main():
     bufs = [torch.empty(gib, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(4)]
     rates = {}
     for mode, name, moved in ((0, "read_only_GBs", gib), (1, "write_only_GBs", gib), (2, "copy_GBs", 2 * gib)):
-        for i in range(3):
-            _capi.probe_stream(bufs[i % 4].data_ptr(), bufs[(i + 1) % 4].data_ptr(), gib, mode, stream.cuda_stream)
-        torch.cuda.synchronize(dev)
-        ev4 = torch.cuda.Event(enable_timing=True)
-        ev5 = torch.cuda.Event(enable_timing=True)
-        ev4.record(stream)
-        for i in range(12):
-            _capi.probe_stream(bufs[i % 4].data_ptr(), bufs[(i + 1) % 4].data_ptr(), gib, mode, stream.cuda_stream)
-        ev5.record(stream)
-        torch.cuda.synchronize(dev)
-        rates[name] = moved / (ev4.elapsed_time(ev5) * 1e-3 / 12) / 1e9
+        us = timed(lambda i, mode=mode: _capi.probe_stream(bufs[i % 4].data_ptr(), bufs[(i + 1) % 4].data_ptr(), gib, mode,
+                                                           stream.cuda_stream), 12, 3)
+        rates[name] = moved / (us * 1e-6) / 1e9
     del bufs
     info = _capi.device_info()
     out["device"] = {"name": torch.cuda.get_device_properties(dev).name, "compute_units": info.compute_units,
@@ -255,7 +330,12 @@ def main():
                      "peak_transfers_per_clock": (HBM_PEAK_GBS * 1e9 * 8 / (info.memory_bus_bits * info.memory_clock_khz * 1e3)
                                                   if info.memory_bus_bits and info.memory_clock_khz else None)}
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(torch, cfg)
+        out["cpu_baseline"] = cpu_baseline(torch, cfg, first, kernel_out)
+        bad = [k for k, same in out["cpu_baseline"]["kernel_outputs_bit_identical_to_oracle"].items() if not same]
+        if bad:
+            print(json.dumps(out))
+            print("bench.py: kernel outputs differ from the oracle: %s" % ", ".join(bad), file=sys.stderr)
+            sys.exit(3)
     print(json.dumps(out))
 
 

@@ -183,6 +183,11 @@ int tde_reduce_rms_static_stage(const tde_problem *problem, const tde_buffers *b
    measuring the device's practical streaming ceiling.  No counterpart in the reference. */
 int tde_probe_copy(void *dst, const void *src, int64_t bytes, void *hip_stream);
 
+/* Measurement aid: enqueue one empty kernel (one wavefront, no memory access).  Back-to-back calls timed on a stream
+   give the cost of a dispatch itself, the floor under the small, latency-bound problems.  No counterpart in the
+   reference. */
+int tde_probe_launch(void *hip_stream);
+
 /* Measurement aid: the device's practical streaming rates.  mode 0 reads `bytes` from src (dst, at least 16
    bytes, is not written for any realistic data), 1 writes `bytes` to dst (src is not read), 2 copies; one
    workgroup per 4 KiB, no loop.  `bytes` a multiple of 16.  No counterpart in the reference. */
@@ -194,6 +199,13 @@ int tde_probe_stream(void *dst, const void *src, int64_t bytes, int32_t mode, vo
    q_out.  Fused algorithm only (TDE_EALGO for the staged ones).  Timing it next to tde_reduce_rms shows how
    far the kernel is from what its access pattern alone achieves.  No counterpart in the reference. */
 int tde_probe_rows(const tde_problem *problem, const tde_buffers *buffers, void *hip_stream);
+
+/* tde_probe_rows with parts of the traffic switched off, to measure what each part of the access pattern costs on its
+   own in the same process as the kernel: `parts` is a bit set -- 1 read the N partial rows and the residual row,
+   2 write the T-typed output rows (residual_out, and norm_out where the problem writes it), 4 write the code rows;
+   7 is tde_probe_rows.  With bit 1 clear nothing is read (the rows written are a thread pattern); with bits 2 and 4
+   clear nothing is written for any realistic data.  TDE_EINVAL outside 1..7.  No counterpart in the reference. */
+int tde_probe_rows_parts(const tde_problem *problem, const tde_buffers *buffers, int32_t parts, void *hip_stream);
 
 /* Properties of the current device as the HIP runtime reports them, for printing next to measured rates:
    compute units, memory clock (kHz), memory bus width (bits; 0 where the runtime reports none) and total

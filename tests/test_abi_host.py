@@ -173,6 +173,23 @@ def test_torch_schemas_match_reference():
     assert inspect.signature(tde.setup_env).parameters["max_size_in_bytes"].default == 8192 * 16384
 
 
+def test_reference_package_name_resolves_to_this_build():
+    """A caller written against the reference does `import torch_dist_ext` (test/test_all_reduce_fusion.py:8) and
+    the reference loads `<parent of the package>/libtorch_dist_ext.so` (torch_dist_ext/__init__.py:8-12)."""
+    import importlib
+    import os
+    import torch_dist_ext
+    import torch_dist_ext_amd
+    assert torch_dist_ext is torch_dist_ext_amd
+    assert importlib.import_module("torch_dist_ext") is torch_dist_ext_amd
+    for name in ("CommWorkspace", "allreduce_rms_fusion_impl", "CommProcess", "setup_env", "get_workspace", "allreduce_rms"):
+        assert hasattr(torch_dist_ext, name), name
+    assert torch_dist_ext.allreduce_rms is torch.ops.torch_dist_ext.allreduce_rms
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    assert os.path.samefile(torch_dist_ext.filename, os.path.join(root, "libtorch_dist_ext.so"))
+    assert os.path.isdir(os.path.join(root, "torch_dist_ext"))   # the directory whose name the loader rule starts from
+
+
 def test_fake_tensor_shapes():
     import torch_dist_ext_amd as tde
     from torch._subclasses.fake_tensor import FakeTensorMode

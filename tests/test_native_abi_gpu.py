@@ -1,5 +1,5 @@
 """GPU: the C ABI driven from a plain C++ program (tests/native/unit_test_abi.cpp, built by
-torch_dist_ext_amd/_build.py), over the shape grid of the reference's native test (test/unit_test.cpp:322-323)."""
+tests/native/build_native.py), over the shape grid of the reference's native test (test/unit_test.cpp:322-323)."""
 import os
 import subprocess
 
@@ -11,7 +11,7 @@ BINARY = os.path.join(os.path.dirname(os.path.abspath(__file__)), "native", "uni
 
 
 def test_native_unit_test(cuda_device):
-    assert os.path.exists(BINARY), "build first: python torch_dist_ext_amd/_build.py"
+    assert os.path.exists(BINARY), "build first: python tests/native/build_native.py"
     proc = subprocess.run([BINARY], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=110)
     print(proc.stdout, flush=True)
     assert proc.returncode == 0, proc.stdout

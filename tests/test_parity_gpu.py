@@ -342,9 +342,25 @@ def test_static_scale_fp8(cuda_device, dtype, scale):
     assert "scale" not in got
     check_against_oracle({k: got[k] for k in ("residual_out", "norm_out")}, want, "none", gamma=g, eps=1e-6)
     assert bits_equal(got["q"], eager.quant_fp8_static(got["norm_out"], scale))
-    assert int(ulp_distance(got["q"], want["q"]).max()) <= 1
+    assert bits_equal(got["q"], want["q"])
     got2 = run_hip(p, r, g, 1e-6, "fp8_static", static_scale=scale, write_norm=False)
     assert bits_equal(got2["q"], got["q"])
+
+
+@pytest.mark.parametrize("dtype,gscale,scale", [(torch.float32, 1e30, 1e-9), (torch.bfloat16, 1e30, 1e-9), (torch.float32, 1e25, 3e-17)])
+def test_static_scale_quotient_beyond_fp32_range(cuda_device, dtype, gscale, scale):
+    """Normed values around 1e30 (or 1e25) divided by a static scale of 1e-9 (3e-17) leave the fp32 range: the codes
+    must saturate with the value's own sign (0x7E / 0xFE), exactly as the oracle's clamp does."""
+    p, r, g = eager.make_inputs(4, 9, 1024, torch.float32, 1.0, seed=43)
+    p, r, g = p.to(dtype), r.to(dtype), (g * gscale).to(dtype)
+    want = eager.reduce_rms(p, r, g, 1e-6, "fp8_static", static_scale=scale)
+    got = run_hip(p, r, g, 1e-6, "fp8_static", static_scale=scale)
+    assert bits_equal(got["norm_out"], want["norm_out"])
+    assert bits_equal(got["q"], want["q"])
+    codes = got["q"].view(torch.uint8)
+    nonzero = want["norm_out"].float() != 0
+    assert bool(((codes[nonzero] & 0x7F) == 0x7E).all())
+    assert bool(((codes >> 7).bool() == (want["norm_out"].float() < 0))[nonzero].all())
 
 
 def test_static_scale_is_validated(cuda_device):

@@ -198,3 +198,73 @@ def test_ops_under_default_torch_compile(tde, cuda_device):
     assert torch.equal(ro1.cpu(), want["residual_out"].float() + 1)
     e_deq, e_ro1 = step(x, rd, gd, ws)
     assert torch.equal(deq, e_deq) and torch.equal(ro1, e_ro1)
+
+
+def test_reference_test_body_under_the_reference_package_name(cuda_device):
+    """The body of the reference's worker (test/test_all_reduce_fusion.py:42-61) with its own import line,
+    `import torch_dist_ext`, on one GPU: setup_env, get_workspace, allreduce_rms, compared with the eager
+    composition of the same file (:17-28, :72-76).  Only the peers' partials are placed by hand."""
+    import torch_dist_ext
+    world_size, num_tokens, hidden_dim, eps, rank = 4, 129, 1024, 1e-6, 0
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(99)
+    allreduce_in = torch.randn((world_size, num_tokens, hidden_dim), generator=g).to(dtype)
+    residual_in = torch.randn((num_tokens, hidden_dim), generator=g).to(dtype)
+    weight = torch.randn((hidden_dim,), generator=g).to(dtype)
+    want = eager.reduce_rms(allreduce_in, residual_in, weight, eps)
+    torch_dist_ext.setup_env(rank, world_size)
+    for r in range(1, world_size):
+        torch_dist_ext.set_peer_partial(r, allreduce_in[r].to(cuda_device))
+    local_in = allreduce_in[rank].to(cuda_device)
+    workspace = torch_dist_ext.get_workspace(local_in)
+    norm_out, residual_out = torch_dist_ext.allreduce_rms(rank, world_size, local_in, residual_in.to(cuda_device),
+                                                          weight.to(cuda_device), eps, workspace)
+    torch.cuda.synchronize()
+    check_against_oracle({"norm_out": norm_out.cpu(), "residual_out": residual_out.cpu()}, want, "none", gamma=weight, eps=eps)
+
+
+def test_torch_ops_inside_a_hip_graph(tde, cuda_device):
+    """get_workspace outside the capture, allreduce_rms and allreduce_rms_quant inside it; the graph is replayed
+    with new input contents several times, with eager work and synchronizations in between, and every replay is
+    compared with the oracle."""
+    world_size, tokens, hidden, eps, rank = 4, 96, 2048, 1e-5, 2
+    tde.setup_env(rank, world_size, max_size_in_bytes=tokens * hidden * 2)
+    p, r, g = eager.make_inputs(world_size, tokens, hidden, torch.bfloat16, 0.5, seed=41)
+    local_in = p[rank].to(cuda_device)
+    res_in, gamma = r.to(cuda_device), g.to(cuda_device)
+    peers = {k: tde.peer_partial(k, local_in) for k in range(world_size) if k != rank}
+    for k, t in peers.items():
+        t.copy_(p[k].to(cuda_device))
+    ws = tde.get_workspace(local_in)          # uploads the pointer table once, outside the capture
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):              # warm-up on the capture stream
+        tde.allreduce_rms(rank, world_size, local_in, res_in, gamma, eps, ws)
+        torch.ops.torch_dist_ext.allreduce_rms_quant(rank, world_size, local_in, res_in, gamma, eps, ws, tde.QUANT_FP8_TOKEN, False)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        norm_out, residual_out = tde.allreduce_rms(rank, world_size, local_in, res_in, gamma, eps, ws)
+        q, scale, residual_out2, _ = torch.ops.torch_dist_ext.allreduce_rms_quant(
+            rank, world_size, local_in, res_in, gamma, eps, ws, tde.QUANT_FP8_TOKEN, False)
+    for replay in range(4):
+        p2, r2, _ = eager.make_inputs(world_size, tokens, hidden, torch.bfloat16, 0.5, seed=50 + replay)
+        local_in.copy_(p2[rank].to(cuda_device))
+        res_in.copy_(r2.to(cuda_device))
+        for k, t in peers.items():
+            t.copy_(p2[k].to(cuda_device))
+        for t in (norm_out, residual_out, residual_out2):
+            t.fill_(float("nan"))
+        q.view(torch.uint8).fill_(0xFF)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = eager.reduce_rms(p2, r2, g, eps, "fp8_token")
+        check_against_oracle({"norm_out": norm_out.cpu(), "residual_out": residual_out.cpu()}, want, "none", gamma=g, eps=eps)
+        assert bits_equal(residual_out2.cpu(), want["residual_out"])
+        assert bits_equal(q.cpu(), want["q"]) and bits_equal(scale.cpu(), want["scale"])
+        # eager work between replays
+        eager_norm, _ = tde.allreduce_rms(rank, world_size, local_in, res_in, gamma, eps, ws)
+        assert bits_equal(eager_norm.cpu(), want["norm_out"])
+

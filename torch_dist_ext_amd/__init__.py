@@ -22,7 +22,8 @@ from ._capi import (ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, ALGO_STAGED_OWNED, QUANT
                     QUANT_NONE, QUANT_GROUP)
 
 this_dir = os.path.dirname(os.path.abspath(__file__))
-filename = os.path.join(this_dir, "libtorch_dist_ext.so")
+# where the reference's loader looks (torch_dist_ext/__init__.py:8-12): beside the package directory
+filename = os.path.join(os.path.dirname(this_dir), "libtorch_dist_ext.so")
 if not (os.path.exists(filename) and os.path.exists(_capi.LIB_PATH)):
     raise ImportError(
         "torch_dist_ext_amd: %s / %s not built. Run `python torch_dist_ext_amd/_build.py` "

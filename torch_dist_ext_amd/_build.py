@@ -2,9 +2,10 @@
 
   libtde_hip.so          hipcc, gfx950 only: the HIP kernels and the C ABI (include/tde_abi.h)
   libtorch_dist_ext.so   host compiler only: the torch operator/class registration, linked against
-                         libtde_hip.so (the name the reference's package loads, torch_dist_ext/__init__.py:8-12)
+                         libtde_hip.so.  Name and place are the reference loader's (torch_dist_ext/__init__.py:8-12:
+                         `<parent of the package directory>/lib<package>.so`), i.e. the repository root.
 
-Both land next to this file so they travel with the source tree.
+libtde_hip.so lands next to this file, libtorch_dist_ext.so one level up; both travel with the source tree.
 Run as `python torch_dist_ext_amd/_build.py` (by path: importing the package needs the libraries
 this script produces).
 """
@@ -19,7 +20,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 INCLUDE = os.path.join(ROOT, "include")
 OBJ_DIR = os.path.join(PKG_DIR, "build")
 HIP_LIB = os.path.join(PKG_DIR, "libtde_hip.so")
-TORCH_LIB = os.path.join(PKG_DIR, "libtorch_dist_ext.so")
+TORCH_LIB = os.path.join(ROOT, "libtorch_dist_ext.so")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 HIP_SOURCES = ["tde_abi.hip", "tde_rows_bf16.hip", "tde_rows_f16.hip", "tde_rows_f32.hip", "tde_rows_f64.hip", "tde_probe.hip"]
@@ -75,7 +76,7 @@ def build_torch(verbose=False):
     ] + inc + [
         os.path.join(CSRC, "tde_torch.cpp"), "-o", TORCH_LIB,
         "-L", PKG_DIR, "-ltde_hip", "-L", torch_lib_dir, "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip",
-        "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib_dir, "-Wl,--no-as-needed",
+        "-Wl,-rpath,$ORIGIN/torch_dist_ext_amd", "-Wl,-rpath," + torch_lib_dir, "-Wl,--no-as-needed",
     ]
     out = _run(cmd)
     if verbose and out.strip():
@@ -83,27 +84,9 @@ def build_torch(verbose=False):
     return TORCH_LIB
 
 
-def build_native_test(verbose=False):
-    """tests/native/unit_test_abi: a C++ program that drives the C ABI without Python or torch and checks
-    it against the oracle's C restatement (linked in as the checker)."""
-    hipcc = os.path.join(ROCM, "bin", "hipcc")
-    src = os.path.join(ROOT, "tests", "native", "unit_test_abi.cpp")
-    out = os.path.join(ROOT, "tests", "native", "unit_test_abi")
-    oracle_dir = os.path.join(ROOT, "oracle")
-    _run(["make", "-C", oracle_dir, "libtde_oracle.so"])
-    cmd = [hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", "-I", INCLUDE, src, "-o", out,
-           "-L", PKG_DIR, "-ltde_hip", "-L", oracle_dir, "-ltde_oracle",
-           "-Wl,-rpath,$ORIGIN/../../torch_dist_ext_amd", "-Wl,-rpath,$ORIGIN/../../oracle"]
-    o = _run(cmd)
-    if verbose and o.strip():
-        print(o)
-    return out
-
-
 def build_all(verbose=False):
     build_hip(verbose)
     build_torch(verbose)
-    build_native_test(verbose)
     return HIP_LIB, TORCH_LIB
 
 

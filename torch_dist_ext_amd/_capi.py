@@ -20,7 +20,7 @@ ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, ALGO_STAGED_OWNED = 0, 1, 2, 3
 EXPORTS = (
     "tde_abi_version", "tde_status_string", "tde_last_hip_error", "tde_plan", "tde_reduce_rms", "tde_stage_reduce", "tde_stage_norm",
     "tde_reduce_rms_static_stage",
-    "tde_probe_copy", "tde_probe_stream", "tde_probe_rows", "tde_device_info",
+    "tde_probe_copy", "tde_probe_launch", "tde_probe_stream", "tde_probe_rows", "tde_probe_rows_parts", "tde_device_info",
     "tde_workspace_create", "tde_workspace_destroy", "tde_workspace_slot", "tde_workspace_stage",
     "tde_workspace_slot_bytes", "tde_workspace_nranks", "tde_workspace_fill_table",
 )
@@ -87,6 +87,10 @@ def load():
     for fn in (lib.tde_stage_reduce, lib.tde_stage_norm, lib.tde_probe_rows, lib.tde_reduce_rms_static_stage):
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(Problem), ctypes.POINTER(Buffers), ctypes.c_void_p]
+    lib.tde_probe_rows_parts.restype = ctypes.c_int
+    lib.tde_probe_rows_parts.argtypes = [ctypes.POINTER(Problem), ctypes.POINTER(Buffers), ctypes.c_int32, ctypes.c_void_p]
+    lib.tde_probe_launch.restype = ctypes.c_int
+    lib.tde_probe_launch.argtypes = [ctypes.c_void_p]
     lib.tde_probe_copy.restype = ctypes.c_int
     lib.tde_probe_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
     lib.tde_probe_stream.restype = ctypes.c_int

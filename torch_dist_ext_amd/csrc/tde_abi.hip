@@ -178,6 +178,9 @@ __global__ void __launch_bounds__(256) copy_kernel(const void *src, void *dst, i
     }
 }
 
+// Nothing: what one dispatch costs when it does no work.
+__global__ void __launch_bounds__(64) empty_kernel() {}
+
 // Streaming-rate probes: one 256-thread workgroup per 4 KiB, no loop (the shape that measured fastest for
 // both directions).  MODE 0 reads only (the loaded words feed a store that never executes for real data),
 // 1 writes only, 2 copies.
@@ -245,6 +248,12 @@ int tde_probe_copy(void *dst, const void *src, int64_t bytes, void *hip_stream) 
     return e == hipSuccess ? TDE_OK : hip_fail(e);
 }
 
+int tde_probe_launch(void *hip_stream) {
+    hipLaunchKernelGGL(empty_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(hip_stream));
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? TDE_OK : hip_fail(e);
+}
+
 int tde_probe_stream(void *dst, const void *src, int64_t bytes, int32_t mode, void *hip_stream) {
     if (dst == nullptr || src == nullptr || bytes < 0 || bytes % 16 != 0 || mode < 0 || mode > 2) return TDE_EINVAL;
     if (!aligned16(dst) || !aligned16(src)) return TDE_EALIGN;
@@ -306,7 +315,7 @@ int tde_plan(const tde_problem *problem, tde_plan_out *plan) {
 namespace {
 enum : int { kPhaseReduce = 1, kPhaseNorm = 2, kTrafficOnly = 4 };
 
-int run_phases(const tde_problem *p, const tde_buffers *b, void *hip_stream, int phases) {
+int run_phases(const tde_problem *p, const tde_buffers *b, void *hip_stream, int phases, int probe_parts = 7) {
     tde::Geometry g{};
     const int st = validate(p, &g);
     if (st != TDE_OK) return st;
@@ -361,6 +370,7 @@ int run_phases(const tde_problem *p, const tde_buffers *b, void *hip_stream, int
     a.eps = p->eps;
     a.hidden_f = (float)p->hidden;
     a.static_scale = p->static_scale;
+    a.probe_parts = probe_parts;
 
     int n = p->nranks;
     hipError_t e = hipSuccess;
@@ -436,6 +446,11 @@ int tde_reduce_rms_static_stage(const tde_problem *p, const tde_buffers *b, void
 
 int tde_probe_rows(const tde_problem *p, const tde_buffers *b, void *hip_stream) {
     return run_phases(p, b, hip_stream, kTrafficOnly);
+}
+
+int tde_probe_rows_parts(const tde_problem *p, const tde_buffers *b, int32_t parts, void *hip_stream) {
+    if (parts < 1 || parts > 7) return TDE_EINVAL;
+    return run_phases(p, b, hip_stream, kTrafficOnly, parts);
 }
 
 // ---- emulated peer workspace ----------------------------------------------------------------

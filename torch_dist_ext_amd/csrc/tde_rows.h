@@ -55,6 +55,7 @@ struct RowArgs {
     float eps;
     float hidden_f;
     float static_scale;
+    int32_t probe_parts; // traffic skeleton only: bit 0 read the inputs, bit 1 write the T-typed rows, bit 2 write the code rows
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -303,12 +304,20 @@ __device__ __forceinline__ float sumsq_torch_order(float *lds_img, float *lds_bs
     if (waves_per_row > 1) __syncthreads(); else wave_lds_fence();
 
     // Lane 4m + k of every wavefront sums the blocks of chain (m, k); the quad then holds the four chains of m.
-    float v[16];
-#pragma unroll
-    for (int b2 = 0; b2 < 16; ++b2) v[b2] = bs[(b2 < blocks ? b2 : 0) * 32 + cl];
     float chain = 0.0f;
+    if (blocks == 16) {
+        float v[16];
 #pragma unroll
-    for (int b2 = 0; b2 < 16; ++b2) chain += (b2 < blocks) ? v[b2] : 0.0f;
+        for (int b2 = 0; b2 < 16; ++b2) v[b2] = bs[b2 * 32 + cl];
+#pragma unroll
+        for (int b2 = 0; b2 < 16; ++b2) chain += v[b2];
+    } else {
+        float v[16];
+#pragma unroll
+        for (int b2 = 0; b2 < 16; ++b2) v[b2] = bs[(b2 < blocks ? b2 : 0) * 32 + cl];
+#pragma unroll
+        for (int b2 = 0; b2 < 16; ++b2) chain += (b2 < blocks) ? v[b2] : 0.0f;
+    }
     const int m = cl >> 2;
     float p = quad_bcast<0x00>(chain);
     for (int l = 0; l < L; ++l) p += img[8 * (4 * I + l) + m];
@@ -637,6 +646,14 @@ __global__ void __launch_bounds__(1024 / VPT)
                 E::unpack(yraw[j], y);
                 const float div = (scale[j] > 0.0f) ? scale[j] : 1.0f;
                 const float rcp = 1.0f / div;
+                if constexpr (Q == TDE_QUANT_FP8_STATIC) {
+                    // A caller's scale can be far below the row's values (the dynamic scales cannot: |y| <= QMAX * scale).
+                    // Beyond twice the largest code the quotient clamps to QMAX whatever it is, so y is cut there: the
+                    // product y * rcp then stays finite and the correction below never sees inf - inf.
+                    const float ymax = (div < 0x1p60f) ? 2.0f * QMAX * div : 3.0e38f;
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) y[i] = fminf(fmaxf(y[i], -ymax), ymax);
+                }
                 // One wavefront-uniform decision, so the common path carries no per-lane branch.
                 const bool unsafe = !(div > 0x1p-60f && div < 0x1p60f);
                 if (__builtin_amdgcn_ballot_w64(unsafe) == 0) {

@@ -130,12 +130,13 @@ public:
     // src/ops/all_reduce_fusion.cpp:159-173): no host-to-device copy in steady state, which also
     // keeps the call legal while a HIP graph is being captured.
     Tensor get_workspace(const Tensor &ref) {
-        if (table_.defined() && table_.device() == ref.device()) return table_;
+        TORCH_CHECK(ref.is_cuda() && ref.device().index() == device_,
+                    "get_workspace: ref must live on the workspace's GPU (device ", device_, "): the table holds that device's pointers");
+        if (table_.defined()) return table_;
         const int64_t entries = 3 * world_size_ + 5;
         auto host = at::empty({entries * (int64_t)sizeof(void *)}, at::TensorOptions().dtype(at::kByte).device(at::kCPU));
         check_status(tde_workspace_fill_table(ws_, reinterpret_cast<void **>(host.data_ptr()), (int32_t)entries),
                      "get_workspace");
-        if (table_.defined()) unregister_table(table_.data_ptr());
         table_ = host.to(ref.device());
         register_table(table_.data_ptr(), size_in_bytes_);
         return table_;
@@ -257,6 +258,8 @@ void use_table(Call &c, int64_t rank, int64_t nranks, const Tensor &allreduce_in
     const int64_t slot_bytes = table_slot_bytes(workspace.data_ptr());
     TORCH_CHECK(slot_bytes >= 0, "workspace is not a pointer table handed out by a live CommWorkspace's get_workspace "
                                  "(pass that tensor itself, not a copy)");
+    TORCH_CHECK(allreduce_in.is_cuda() && allreduce_in.device() == workspace.device(),
+                "allreduce_in must live on the workspace's GPU: the pointer table holds that device's addresses");
     const int64_t bytes = allreduce_in.numel() * (int64_t)allreduce_in.element_size();
     TORCH_CHECK(bytes <= slot_bytes, "allreduce_in has ", bytes, " bytes but the workspace slots hold ", slot_bytes,
                 "; create the workspace (setup_env) with a larger size");
