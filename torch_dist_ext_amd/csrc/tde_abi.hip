@@ -108,14 +108,17 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     // Vectors per thread.  Four vectors per thread (small workgroups, many loads in flight per thread,
     // few wavefronts to synchronize per row) win where they fill their lanes: rows of 896+ vectors, and
     // rows of exactly 256/512/1024 vectors (one, two or four full wavefronts per row); measured on
-    // MI355X across hidden 2048..8192, the other sizes are as fast or faster with one vector per thread,
-    // as are 512-vector rows with four or fewer partials.
+    // MI355X across hidden 1024..8192, the other sizes are as fast or faster with one vector per thread,
+    // as are 512-vector rows with four or fewer partials.  Rows of 640 vectors (hidden 5120 in a 2-byte type)
+    // with four or fewer partials are the exception: 2.5 % (32768 rows) to 5 % (4096 rows) faster with four.
     int vpt = 1;
     if (nvec >= 896) {
-        // Few rows are latency-bound and the widest row groups have the shortest dependent chain; in between,
-        // two vectors per thread measure 1-4 % faster than either neighbour.
-        vpt = p->tokens >= 768 ? 4 : (p->tokens >= 160 ? 2 : 1);
+        // Few rows are latency-bound and the widest row groups have the shortest dependent chain; from 256 rows
+        // up four vectors per thread are 8-13 % faster than one or two (8 partials, hidden 8192).
+        vpt = p->tokens >= 256 ? 4 : (p->tokens >= 128 ? 2 : 1);
     } else if ((nvec == 256 || (nvec == 512 && p->nranks >= 8)) && p->tokens >= 1024) {
+        vpt = 4;
+    } else if (nvec == 640 && p->nranks <= 4 && p->tokens >= 2048) {
         vpt = 4;
     }
     if (p->tune_vecs_per_thread != 0) {
