@@ -217,3 +217,27 @@ def test_cpu_tensors_are_rejected_not_silently_computed():
     with pytest.raises((RuntimeError, NotImplementedError)):
         tde.allreduce_rms_fusion_impl(0, 2, x, x, g, torch.empty_like(x), torch.empty_like(x), 1e-6,
                                       torch.zeros(88, dtype=torch.uint8))
+
+
+def test_bench_draws_the_configurations_seeded_inputs():
+    """bench.py checks the kernel's outputs for its first input set against the oracle; that set must be the
+    configuration's seeded inputs (the same tensors the parity tests use)."""
+    import importlib.util
+    import os
+    from oracle import eager
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("tde_bench", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    got = bench.seeded_cpu_inputs(torch, bench.BENCH_CONFIGS["c2"])
+    want = eager.make_config("c2")[:3]
+    for g, w in zip(got, want):
+        assert torch.equal(g.view(torch.int16), w.view(torch.int16))
+    cfg = list(bench.BENCH_CONFIGS["c5"])
+    cfg[1] = 64                                    # c5 at 64 rows: the outlier channels and the fp16 cast
+    got = bench.seeded_cpu_inputs(torch, tuple(cfg))
+    want = eager.make_config("c5", tokens=64)[:3]
+    for g, w in zip(got, want):
+        assert torch.equal(g.view(torch.int16), w.view(torch.int16))
+    assert bench.BENCH_CONFIGS["c3"][:3] == (8, 2048, 8192) and bench.BENCH_CONFIGS["c3"][5] == eager.CONFIGS["c3"][5]
+    assert len(bench.kernel_sources_sha256()) == 64
