@@ -652,3 +652,46 @@ def test_committed_golden_fixtures_through_the_kernel(cuda_device, name):
     if quant != "none":
         assert np.array_equal(got["q"].view(torch.uint8).numpy(), d[name + "/q"])
         assert np.array_equal(got["scale"].numpy().view(np.uint32), d[name + "/scale"].view(np.uint32))
+
+
+def test_more_than_2_to_the_31_elements_per_buffer(cuda_device):
+    """270 000 rows of 8192 bf16 are 2.2e9 elements and 4.4 GB per buffer: byte offsets and element counts beyond
+    32 bits (the reference indexes with int, src/common/all_reduce_fusion_impl.h:304).  The rows at the start, around
+    element 2^31 (row 262 144) and at the end must equal what the same kernel computes for those rows alone, which in
+    turn is checked against the oracle."""
+    n, t, h, eps = 2, 270000, 8192, 1e-5
+    dev = cuda_device
+    gen = torch.Generator(device=dev).manual_seed(5)
+    parts = []
+    for _ in range(n):
+        p = torch.empty((t, h), dtype=torch.bfloat16, device=dev)
+        for lo in range(0, t, 30000):       # in pieces: no fp32 copy of the whole buffer
+            hi = min(t, lo + 30000)
+            p[lo:hi] = (torch.randn((hi - lo, h), generator=gen, device=dev) * 0.5).to(torch.bfloat16)
+        parts.append(p)
+    res = torch.empty((t, h), dtype=torch.bfloat16, device=dev)
+    for lo in range(0, t, 30000):
+        hi = min(t, lo + 30000)
+        res[lo:hi] = torch.randn((hi - lo, h), generator=gen, device=dev).to(torch.bfloat16)
+    gamma = (torch.rand((h,), generator=gen, device=dev) + 0.5).to(torch.bfloat16)
+    res_out = torch.empty_like(res)
+    q = torch.empty((t, h), dtype=torch.uint8, device=dev)
+    scale = torch.empty((t,), dtype=torch.float32, device=dev)
+    for buf in (res_out, q, scale):
+        buf.view(torch.uint8).fill_(0xFF)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    prob = _capi.make_problem(_capi.BF16, n, t, h, eps, quant=_capi.QUANT_FP8_TOKEN, write_norm=0)
+    assert _capi.plan(prob).grid_blocks == t
+    print("case 2^31 elements", t, h, flush=True)
+    _capi.reduce_rms(prob, [p.data_ptr() for p in parts], res.data_ptr(), res_out.data_ptr(), gamma.data_ptr(),
+                     q_out=q.data_ptr(), scale_out=scale.data_ptr(), stream=stream)
+    torch.cuda.synchronize(dev)
+    boundary = (1 << 31) // h
+    for lo, hi in ((0, 40), (boundary - 20, boundary + 20), (t - 40, t)):
+        cp = torch.stack([p[lo:hi] for p in parts]).cpu()
+        want = eager.reduce_rms(cp, res[lo:hi].cpu(), gamma.cpu(), eps, "fp8_token")
+        assert bits_equal(res_out[lo:hi].cpu(), want["residual_out"]), (lo, hi)
+        assert bits_equal(q[lo:hi].cpu(), want["q"]), (lo, hi)
+        assert bits_equal(scale[lo:hi].cpu(), want["scale"]), (lo, hi)
+    # every row was written (no 0xFF fill left in the scales) and rows far apart differ
+    assert bool(torch.isfinite(scale).all()) and bool((scale > 0).all())
