@@ -695,3 +695,29 @@ def test_more_than_2_to_the_31_elements_per_buffer(cuda_device):
         assert bits_equal(scale[lo:hi].cpu(), want["scale"]), (lo, hi)
     # every row was written (no 0xFF fill left in the scales) and rows far apart differ
     assert bool(torch.isfinite(scale).all()) and bool((scale > 0).all())
+
+
+SUM_ORDER_HIDDEN = {
+    # vectors of 8 floats V = hidden // 8: left-over vectors V % 4, left-over scalars hidden % 8, a last block shorter
+    # than 16 steps ((V // 4) % 16), no full step at all (V < 4), fewer than 8 floats
+    torch.bfloat16: [8, 16, 24, 32, 40, 72, 120, 128, 136, 264, 504, 520, 1032, 2040, 2056, 4104, 6152, 8184],
+    torch.float16: [8, 56, 520, 4088],
+    torch.float32: [4, 8, 12, 20, 28, 36, 100, 132, 516, 1028, 2052, 4092],
+    torch.float64: [2, 4, 6, 8, 10, 14, 18, 66, 130, 1026, 2046],
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32, torch.float64])
+def test_sum_of_squares_order_at_every_row_shape(cuda_device, dtype):
+    """The kernel's sum of squares follows torch's CPU reduction through every branch of it: left-over vectors and
+    scalars, a short last block, rows without a full step, rows shorter than one vector.  Normed rows (and int8 codes
+    and scales where the type has them) must be bit-identical to the oracle's at each of these row lengths, with one,
+    several and many rows per workgroup."""
+    for hidden in SUM_ORDER_HIDDEN[dtype]:
+        for rows_per_block in (0, 1):
+            p, r, g = eager.make_inputs(2, 37, hidden, dtype, 1.0, seed=hidden)
+            quant = "int8_token" if dtype in (torch.bfloat16, torch.float16, torch.float32) else "none"
+            print("case sum-order", dtype, hidden, rows_per_block, flush=True)
+            want = eager.reduce_rms(p, r, g, 1e-6, quant)
+            got = run_hip(p, r, g, 1e-6, quant, rows_per_block=rows_per_block)
+            check_against_oracle(got, want, quant, gamma=g, eps=1e-6)
