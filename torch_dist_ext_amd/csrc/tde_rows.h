@@ -281,15 +281,25 @@ __device__ __forceinline__ float sumsq_torch_order(float *lds_img, float *lds_bs
         // Blocks past the row's end sum to zero, and adding zero to a sum of squares changes nothing.
         wave_lds_fence();
         const int w = t >> 6;
-#pragma unroll
-        for (int s = 0; s < (VPT + 1) / 2; ++s) {
-            const int j = (lane >> 5) + 2 * s;
-            if (j < VPT) {
-                const int b = j * waves_per_row + w;
-                int terms = I - 16 * b;
+        if constexpr (VPT == 1) {
+            if (lane < 32) { // one block per wavefront: half of its lanes have a chain
+                int terms = I - 16 * w;
                 terms = terms < 0 ? 0 : (terms > 16 ? 16 : terms);
-                bs[b * 32 + cl] = chain_block_sum<false>(img, b, cl, terms);
+                bs[w * 32 + cl] = chain_block_sum<false>(img, w, cl, terms);
             }
+        } else {
+            // two blocks at a time, one per half of the wavefront; their reads and sums interleave
+            float sum[VPT / 2];
+            int b[VPT / 2];
+#pragma unroll
+            for (int s = 0; s < VPT / 2; ++s) {
+                b[s] = ((lane >> 5) + 2 * s) * waves_per_row + w;
+                int terms = I - 16 * b[s];
+                terms = terms < 0 ? 0 : (terms > 16 ? 16 : terms);
+                sum[s] = chain_block_sum<false>(img, b[s], cl, terms);
+            }
+#pragma unroll
+            for (int s = 0; s < VPT / 2; ++s) bs[b[s] * 32 + cl] = sum[s];
         }
         blocks = cap_blocks;
     } else {
@@ -311,6 +321,12 @@ __device__ __forceinline__ float sumsq_torch_order(float *lds_img, float *lds_bs
         for (int b2 = 0; b2 < 16; ++b2) v[b2] = bs[b2 * 32 + cl];
 #pragma unroll
         for (int b2 = 0; b2 < 16; ++b2) chain += v[b2];
+    } else if (blocks <= 8) {
+        float v[8];
+#pragma unroll
+        for (int b2 = 0; b2 < 8; ++b2) v[b2] = bs[(b2 < blocks ? b2 : 0) * 32 + cl];
+#pragma unroll
+        for (int b2 = 0; b2 < 8; ++b2) chain += (b2 < blocks) ? v[b2] : 0.0f;
     } else {
         float v[16];
 #pragma unroll
