@@ -28,8 +28,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 # (scaled by the plain-copy calibration described there).  They describe the kernels whose sources hash to
 # `sources_sha256`; with any other kernel source the bench line reports traffic as null.
 TRAFFIC = {
-    "sources_sha256": "a41ac5bcd3ca48252cca98b0dd2480a5901ce5eeb4bfc86f55e0550f4aad9cb7",
-    "bytes": {"c2": 11692326, "c3": 352674972, "c4": 765494457, "c5": 2181256730},
+    "sources_sha256": "d45c0fc5e62640228c018c9146942e6cc9be7562c16bca727992fd083f8a0295",
+    "bytes": {"c2": 11688140, "c3": 352679604, "c4": 765490811, "c5": 2181285268},
 }
 
 BENCH_CONFIGS = {
