@@ -721,3 +721,23 @@ def test_sum_of_squares_order_at_every_row_shape(cuda_device, dtype):
             want = eager.reduce_rms(p, r, g, 1e-6, quant)
             got = run_hip(p, r, g, 1e-6, quant, rows_per_block=rows_per_block)
             check_against_oracle(got, want, quant, gamma=g, eps=1e-6)
+
+
+@pytest.mark.parametrize("vecs_per_thread", [0, 1, 2, 4])
+def test_fp16_product_is_rounded_twice_like_the_eager_composition(cuda_device, vecs_per_thread):
+    """T(x * rs) is an fp32 product rounded to fp32 and then to fp16.  An instruction that multiplies and converts in one
+    step rounds the exact product once, which differs where the fp32 product falls on an fp16 rounding boundary.  The
+    inputs hold such elements (counted here with an exact float64 product), and the kernel must still match the oracle
+    bit for bit."""
+    import numpy as np
+    p, r, g = eager.make_inputs(4, 192, 5120, torch.float16, 1.0, seed=77)
+    want = eager.reduce_rms(p, r, g, 1e-6, "none")
+    x = want["residual_out"].float()
+    rs = torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6)
+    twice = (x * rs).to(torch.float16)
+    once = torch.from_numpy((x.double().numpy() * rs.double().numpy()).astype(np.float16))
+    sensitive = int((twice.view(torch.int16) != once.view(torch.int16)).sum())
+    print("case fp16 double rounding: %d of %d elements tell the two apart" % (sensitive, x.numel()), flush=True)
+    assert sensitive >= 8
+    got = run_hip(p, r, g, 1e-6, "none", vecs_per_thread=vecs_per_thread)
+    check_against_oracle(got, want, "none", gamma=g, eps=1e-6)

@@ -28,6 +28,12 @@ HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     # keep fp32 arithmetic scalar: packed fp32 forms are not used on this hardware pool
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # no v_fma_mix*: the compiler folds "multiply in fp32, then convert to fp16" into v_fma_mixlo_f16, which rounds the
+    # exact product once; the operator's contract is the two roundings of the eager composition
+    "-Xclang", "-target-feature", "-Xclang", "-fma-mix-insts",
+    # the kernels fix their own instruction order around the loads (scheduling barriers); the SLP vectorizer
+    # regroups the element-wise arithmetic across them, which costs registers and the overlap with the loads
+    "-fno-slp-vectorize",
     "-Wno-unused-command-line-argument",
 ]
 

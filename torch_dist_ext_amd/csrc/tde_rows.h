@@ -503,8 +503,8 @@ __global__ void __launch_bounds__(1024 / VPT)
     for (int j = 0; j < VPT; ++j) lane_off[j] = (uint32_t)(j * tpr + tid - group * tpr) * 16u;
 // Thread index inside the row group and lane index, rebuilt from the first load offset where they are needed:
 // the thread id itself does not stay in a register through the load phase, which has none to spare.
-#define TDE_T ((int)(lane_off[0] >> 4))
-#define TDE_LANE ((int)(lane_off[0] >> 4) & (kWave - 1))
+#define TDE_T ((int)(lane0 >> 4))
+#define TDE_LANE ((int)(lane0 >> 4) & (kWave - 1))
 
     auto issue_loads = [&](RowLoads<NP, VPT> &d, int64_t row) {
         const uint32_t bytes = (row < a.tokens) ? row_bytes : 0u;
@@ -533,6 +533,13 @@ __global__ void __launch_bounds__(1024 / VPT)
         __builtin_amdgcn_sched_barrier(0);
         gamma_early = __builtin_amdgcn_raw_buffer_load_b128(gamma_rsrc, (int)lane_off[0], 0, kAuxDefault);
     }
+    // From here on only the first offset stays in a register (the compiler cannot see where it came from, so it
+    // keeps neither the thread index nor the other offsets alive through the load phase); the others are one
+    // addition away.
+    uint32_t lane0 = lane_off[0];
+    asm volatile("" : "+v"(lane0));
+    const uint32_t vec_stride = (uint32_t)tpr * 16u;
+#define TDE_OFF(j) (lane0 + (uint32_t)(j) * vec_stride)
 
     {
         const int64_t row = row0 + group;
@@ -543,11 +550,43 @@ __global__ void __launch_bounds__(1024 / VPT)
         // ---- reduce, residual add, sum of squares ------------------------------------------------
         const rsrc_t res_out = row_rsrc(a.residual_out, row_byte, bytes);
         u32x4 xraw[VPT];
+        // With several vectors per thread the partials are summed rank by rank as they arrive (the memory system
+        // returns a wavefront's loads in the order it issued them), so that only the last partial's additions are
+        // left when the row is complete.  The order of every element's additions is the same either way.
+        constexpr bool RANK_MAJOR = (N >= 4 && VPT >= 4);
+        float racc[RANK_MAJOR ? VPT : 1][VEC];
+        if constexpr (RANK_MAJOR) {
+            __builtin_amdgcn_sched_barrier(0);
+            // The first two partials are taken together, vector by vector: their eight sums fit the registers the
+            // two vectors arrived in, so the accumulators cost no registers while all other loads are in flight.
+#pragma unroll
+            for (int j = 0; j < VPT; ++j) {
+                float p0[VEC], p1[VEC];
+                E::unpack(cur.p[j][0], p0);
+                E::unpack(cur.p[j][1], p1);
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) racc[j][i] = (0.0f + p0[i]) + p1[i];
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int r = 2; r < NP; ++r) {
+#pragma unroll
+                for (int j = 0; j < VPT; ++j) {
+                    float p[VEC];
+                    E::unpack(cur.p[j][r], p);
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) racc[j][i] += p[i];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
             float s[VEC];
             if constexpr (N == 0) {
                 E::unpack(cur.p[j][0], s);
+            } else if constexpr (RANK_MAJOR) {
+                E::unpack(E::pack(racc[j]), s);
             } else {
                 float acc[VEC];
 #pragma unroll
@@ -566,7 +605,7 @@ __global__ void __launch_bounds__(1024 / VPT)
 #pragma unroll
             for (int i = 0; i < VEC; ++i) x[i] = s[i] + res[i];
             xraw[j] = E::pack(x);
-            if constexpr (!LATE_RESIDUAL) rsrc_store16(res_out, lane_off[j], xraw[j]);
+            if constexpr (!LATE_RESIDUAL) rsrc_store16(res_out, TDE_OFF(j), xraw[j]);
             E::unpack(xraw[j], x);
             float sq[VEC];
 #pragma unroll
@@ -582,7 +621,7 @@ __global__ void __launch_bounds__(1024 / VPT)
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int j = 0; j < VPT; ++j)
-                gamma_raw[j] = __builtin_amdgcn_raw_buffer_load_b128(gamma_rsrc, (int)lane_off[j], 0, kAuxDefault);
+                gamma_raw[j] = __builtin_amdgcn_raw_buffer_load_b128(gamma_rsrc, (int)TDE_OFF(j), 0, kAuxDefault);
         } else {
             gamma_raw[0] = gamma_early;
         }
@@ -605,7 +644,7 @@ __global__ void __launch_bounds__(1024 / VPT)
             yraw[j] = E::pack(y);
             if constexpr (Q == TDE_QUANT_NONE || WN) {
                 const rsrc_t norm_out = row_rsrc(a.norm_out, row_byte, bytes);
-                rsrc_store16(norm_out, lane_off[j], yraw[j]);
+                rsrc_store16(norm_out, TDE_OFF(j), yraw[j]);
             }
             if constexpr (Q != TDE_QUANT_NONE && Q != TDE_QUANT_FP8_STATIC) {
                 E::unpack(yraw[j], y);
@@ -618,7 +657,7 @@ __global__ void __launch_bounds__(1024 / VPT)
 
         if constexpr (LATE_RESIDUAL && Q == TDE_QUANT_NONE) {
 #pragma unroll
-            for (int j = 0; j < VPT; ++j) rsrc_store16(res_out, lane_off[j], xraw[j]);
+            for (int j = 0; j < VPT; ++j) rsrc_store16(res_out, TDE_OFF(j), xraw[j]);
         }
 
         // ---- dynamic quant epilogue ---------------------------------------------------------------
@@ -636,7 +675,7 @@ __global__ void __launch_bounds__(1024 / VPT)
                     scale[j] = m / QMAX;
                     if ((TDE_LANE & (LANES_PER_GROUP - 1)) == 0)
                         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, scale[j]), sc_out,
-                                                              (int)((lane_off[j] / 16u / LANES_PER_GROUP) * 4u), 0, kAuxDefault);
+                                                              (int)((TDE_OFF(j) / 16u / LANES_PER_GROUP) * 4u), 0, kAuxDefault);
                 }
             } else if constexpr (Q == TDE_QUANT_FP8_STATIC) {
 #pragma unroll
@@ -654,7 +693,7 @@ __global__ void __launch_bounds__(1024 / VPT)
             const rsrc_t q_out = row_rsrc(a.q_out, row * (int64_t)a.hidden, row_ok ? (uint32_t)a.hidden : 0u);
             if constexpr (LATE_RESIDUAL) {
 #pragma unroll
-                for (int j = 0; j < VPT; ++j) rsrc_store16(res_out, lane_off[j], xraw[j]);
+                for (int j = 0; j < VPT; ++j) rsrc_store16(res_out, TDE_OFF(j), xraw[j]);
             }
 #pragma unroll
             for (int j = 0; j < VPT; ++j) {
@@ -684,7 +723,7 @@ __global__ void __launch_bounds__(1024 / VPT)
                     pack_int8<VEC>(q, codes);
                 else
                     pack_fp8<VEC>(q, codes);
-                const uint32_t code_off = (lane_off[j] / 16u) * (uint32_t)VEC;
+                const uint32_t code_off = (TDE_OFF(j) / 16u) * (uint32_t)VEC;
                 if constexpr (VEC == 8) {
                     u32x2 w = {codes[0], codes[1]};
                     __builtin_amdgcn_raw_buffer_store_b64(w, q_out, (int)code_off, 0, kAuxStore);
@@ -697,6 +736,7 @@ __global__ void __launch_bounds__(1024 / VPT)
 }
 #undef TDE_T
 #undef TDE_LANE
+#undef TDE_OFF
 
 // Stage A of the staged algorithm: s = T(sum of partials) for every element, no row structure.
 // One workgroup of 256 threads reduces a contiguous span of 256*U vectors (U vectors per thread,
