@@ -105,21 +105,27 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     int64_t total_bytes = 0; // tokens * hidden * elem must be addressable with 64-bit signed offsets
     if (__builtin_mul_overflow(p->tokens, p->hidden * eb, &total_bytes)) return TDE_ESHAPE;
 
-    // Vectors per thread.  Four vectors per thread (small workgroups, many loads in flight per thread,
-    // few wavefronts to synchronize per row) win where they fill their lanes: rows of 896+ vectors, and
-    // rows of exactly 256/512/1024 vectors (one, two or four full wavefronts per row); measured on
-    // MI355X across hidden 1024..8192, the other sizes are as fast or faster with one vector per thread,
-    // as are 512-vector rows with four or fewer partials.  Rows of 640 vectors (hidden 5120 in a 2-byte type)
-    // with four or fewer partials are the exception: 2.5 % (32768 rows) to 5 % (4096 rows) faster with four.
+    // Vectors per thread, from sweeps on MI355X over hidden 1024..8192, 2/4/8 partials and 256..32768 rows (bf16 and
+    // fp16 agree).  Four vectors per thread (small workgroups, many loads in flight per thread, few wavefronts to
+    // synchronize per row, partials summed while the later ones are still arriving) win on long rows and wherever
+    // eight partials meet full wavefronts; elsewhere one vector per thread is as fast or faster.
     int vpt = 1;
     if (nvec >= 896) {
         // Few rows are latency-bound and the widest row groups have the shortest dependent chain; from 256 rows
-        // up four vectors per thread are 8-13 % faster than one or two (8 partials, hidden 8192).
+        // up four vectors per thread are 4-13 % faster than one (8 partials, hidden 8192).  With two partials
+        // and up to 2048 rows two vectors per thread are another 2-7 % faster.
         vpt = p->tokens >= 256 ? 4 : (p->tokens >= 128 ? 2 : 1);
-    } else if ((nvec == 256 || (nvec == 512 && p->nranks >= 8)) && p->tokens >= 1024) {
-        vpt = 4;
-    } else if (nvec == 640 && p->nranks <= 4 && p->tokens >= 2048) {
-        vpt = 4;
+        if (p->nranks == 2 && p->tokens >= 256 && p->tokens <= 2048) vpt = 2;
+    } else if (nvec == 512 && p->nranks >= 8 && p->tokens >= 1024) {
+        vpt = 4; // 3-4 % over one
+    } else if (nvec == 256 && p->nranks >= 8 && p->tokens >= 2048) {
+        vpt = 4; // 3-6 % over one; with fewer partials or rows one is 3-16 % faster
+    } else if (nvec == 640) {
+        // Ten wavefronts per row leave the compute units unevenly filled: from 640 rows up five wavefronts with two
+        // vectors each are 10-21 % faster until there are enough rows to even that out (2048 with eight partials,
+        // 16384 with four; with two partials one vector per thread stays 16 % behind at any size).
+        const int64_t even_from = p->nranks >= 8 ? 2048 : (p->nranks == 4 ? 16384 : INT64_MAX);
+        if (p->tokens >= 640 && p->tokens < even_from) vpt = 2;
     }
     if (p->tune_vecs_per_thread != 0) {
         if (p->tune_vecs_per_thread != 1 && p->tune_vecs_per_thread != 2 && p->tune_vecs_per_thread != 4) return TDE_EINVAL;

@@ -695,42 +695,55 @@ __global__ void __launch_bounds__(1024 / VPT)
 #pragma unroll
                 for (int j = 0; j < VPT; ++j) rsrc_store16(res_out, TDE_OFF(j), xraw[j]);
             }
+            // One wavefront-uniform decision for all of the thread's vectors, so the common path carries no per-lane
+            // branch: the fast quotient needs every divisor far from the subnormal and overflow ranges.
+            bool unsafe = false;
 #pragma unroll
             for (int j = 0; j < VPT; ++j) {
-                float y[VEC], q[VEC];
-                E::unpack(yraw[j], y);
                 const float div = (scale[j] > 0.0f) ? scale[j] : 1.0f;
-                const float rcp = 1.0f / div;
-                if constexpr (Q == TDE_QUANT_FP8_STATIC) {
-                    // A caller's scale can be far below the row's values (the dynamic scales cannot: |y| <= QMAX * scale).
-                    // Beyond twice the largest code the quotient clamps to QMAX whatever it is, so y is cut there: the
-                    // product y * rcp then stays finite and the correction below never sees inf - inf.
-                    const float ymax = (div < 0x1p60f) ? 2.0f * QMAX * div : 3.0e38f;
-#pragma unroll
-                    for (int i = 0; i < VEC; ++i) y[i] = fminf(fmaxf(y[i], -ymax), ymax);
-                }
-                // One wavefront-uniform decision, so the common path carries no per-lane branch.
-                const bool unsafe = !(div > 0x1p-60f && div < 0x1p60f);
-                if (__builtin_amdgcn_ballot_w64(unsafe) == 0) {
-#pragma unroll
-                    for (int i = 0; i < VEC; ++i) q[i] = fminf(fmaxf(div_shared(y[i], div, rcp), -QMAX), QMAX);
-                } else {
-#pragma unroll
-                    for (int i = 0; i < VEC; ++i) q[i] = fminf(fmaxf(y[i] / div, -QMAX), QMAX);
-                }
-                uint32_t codes[VEC / 4];
-                if constexpr (Q == TDE_QUANT_INT8_TOKEN)
-                    pack_int8<VEC>(q, codes);
-                else
-                    pack_fp8<VEC>(q, codes);
-                const uint32_t code_off = (TDE_OFF(j) / 16u) * (uint32_t)VEC;
-                if constexpr (VEC == 8) {
-                    u32x2 w = {codes[0], codes[1]};
-                    __builtin_amdgcn_raw_buffer_store_b64(w, q_out, (int)code_off, 0, kAuxStore);
-                } else {
-                    __builtin_amdgcn_raw_buffer_store_b32(codes[0], q_out, (int)code_off, 0, kAuxStore);
-                }
+                unsafe = unsafe || !(div > 0x1p-60f && div < 0x1p60f);
             }
+            const bool fast = __builtin_amdgcn_ballot_w64(unsafe) == 0;
+            auto quantize = [&](auto use_fast) {
+#pragma unroll
+                for (int j = 0; j < VPT; ++j) {
+                    float y[VEC], q[VEC];
+                    E::unpack(yraw[j], y);
+                    const float div = (scale[j] > 0.0f) ? scale[j] : 1.0f;
+                    if constexpr (Q == TDE_QUANT_FP8_STATIC) {
+                        // A caller's scale can be far below the row's values (the dynamic scales cannot: |y| <= QMAX *
+                        // scale).  Beyond twice the largest code the quotient clamps to QMAX whatever it is, so y is cut
+                        // there: the product y * rcp then stays finite and the correction never sees inf - inf.
+                        const float ymax = (div < 0x1p60f) ? 2.0f * QMAX * div : 3.0e38f;
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) y[i] = fminf(fmaxf(y[i], -ymax), ymax);
+                    }
+                    if constexpr (decltype(use_fast)::value) {
+                        const float rcp = 1.0f / div;
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) q[i] = fminf(fmaxf(div_shared(y[i], div, rcp), -QMAX), QMAX);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) q[i] = fminf(fmaxf(y[i] / div, -QMAX), QMAX);
+                    }
+                    uint32_t codes[VEC / 4];
+                    if constexpr (Q == TDE_QUANT_INT8_TOKEN)
+                        pack_int8<VEC>(q, codes);
+                    else
+                        pack_fp8<VEC>(q, codes);
+                    const uint32_t code_off = (TDE_OFF(j) / 16u) * (uint32_t)VEC;
+                    if constexpr (VEC == 8) {
+                        u32x2 w = {codes[0], codes[1]};
+                        __builtin_amdgcn_raw_buffer_store_b64(w, q_out, (int)code_off, 0, kAuxStore);
+                    } else {
+                        __builtin_amdgcn_raw_buffer_store_b32(codes[0], q_out, (int)code_off, 0, kAuxStore);
+                    }
+                }
+            };
+            if (fast)
+                quantize(std::true_type{});
+            else
+                quantize(std::false_type{});
         }
     }
 }
