@@ -28,8 +28,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 # (scaled by the plain-copy calibration described there).  They describe the kernels whose sources hash to
 # `sources_sha256`; with any other kernel source the bench line reports traffic as null.
 TRAFFIC = {
-    "sources_sha256": "d45c0fc5e62640228c018c9146942e6cc9be7562c16bca727992fd083f8a0295",
-    "bytes": {"c2": 11688140, "c3": 352679604, "c4": 765490811, "c5": 2181285268},
+    "sources_sha256": "33a97b13590013d364148f65753593367a8bbcb64abe5f0ec9c19b3956b80228",
+    "bytes": {"c2": 11697330, "c3": 352653695, "c4": 765481471, "c5": 2181192678},
 }
 
 BENCH_CONFIGS = {
