@@ -69,3 +69,48 @@ def test_static_stage_limits(cuda_device):
     for algo in (_capi.ALGO_FUSED, _capi.ALGO_STAGED_OWNED):
         prob = _capi.make_problem(_capi.BF16, 8, 16, 1024, 1e-6, algo=algo)
         assert lib.tde_reduce_rms_static_stage(ctypes.byref(prob), ctypes.byref(b), None) == _capi.EALGO
+
+
+def test_static_stage_inside_a_hip_graph(cuda_device):
+    """What the entry point is for: captured in a HIP graph (after one eager call on the device, which looks the
+    array's address up), replayed with new inputs and eager work in between, every replay checked against the oracle."""
+    dev = cuda_device
+    n, t, h = 8, 96, 4096
+    parts = [torch.empty((t, h), dtype=torch.bfloat16, device=dev) for _ in range(n)]
+    res, gamma = torch.empty((t, h), dtype=torch.bfloat16, device=dev), torch.empty((h,), dtype=torch.bfloat16, device=dev)
+    res_out = torch.empty_like(res)
+    q = torch.empty((t, h), dtype=torch.uint8, device=dev)
+    sc = torch.empty((t,), dtype=torch.float32, device=dev)
+    prob = _capi.make_problem(_capi.BF16, n, t, h, 1e-5, quant=_capi.QUANT_FP8_TOKEN)
+
+    def launch(stream):
+        _capi.reduce_rms(prob, [p.data_ptr() for p in parts], res.data_ptr(), res_out.data_ptr(), gamma.data_ptr(),
+                         q_out=q.data_ptr(), scale_out=sc.data_ptr(), stream=stream, phases=("static_stage",))
+
+    def fill(seed):
+        cp, cr, cg = eager.make_inputs(n, t, h, torch.bfloat16, 0.5, seed=seed)
+        for i in range(n):
+            parts[i].copy_(cp[i])
+        res.copy_(cr)
+        gamma.copy_(cg)
+        return cp, cr, cg
+
+    fill(31)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch(side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        launch(torch.cuda.current_stream().cuda_stream)
+    for seed in (32, 33, 34):
+        cp, cr, cg = fill(seed)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = {"residual_out": res_out.cpu(), "q": q.cpu().view(torch.float8_e4m3fn), "scale": sc.cpu()}
+        for v in (res_out, q, sc):
+            v.zero_()                        # eager work between replays
+        torch.cuda.synchronize()
+        check_against_oracle(got, eager.reduce_rms(cp, cr, cg, 1e-5, "fp8_token"), "fp8_token", gamma=cg, eps=1e-5)
