@@ -741,3 +741,32 @@ def test_fp16_product_is_rounded_twice_like_the_eager_composition(cuda_device, v
     assert sensitive >= 8
     got = run_hip(p, r, g, 1e-6, "none", vecs_per_thread=vecs_per_thread)
     check_against_oracle(got, want, "none", gamma=g, eps=1e-6)
+
+
+def test_calls_on_two_streams_at_once(cuda_device):
+    """The launch keeps no state between calls, so calls on different streams with different outputs may overlap: two
+    problems of different shape and mode are launched alternately on two streams, several times over without
+    synchronizing in between, and each is then checked against the oracle."""
+    dev = cuda_device
+    jobs = []
+    for seed, (n, t, h, dtype, dcode, quant, qm) in enumerate([
+            (8, 512, 8192, torch.bfloat16, _capi.BF16, "fp8_token", _capi.QUANT_FP8_TOKEN),
+            (4, 700, 5120, torch.float16, _capi.F16, "int8_token", _capi.QUANT_INT8_TOKEN)]):
+        cp, cr, cg = eager.make_inputs(n, t, h, dtype, 0.5, seed=90 + seed)
+        d = dict(cp=cp, cr=cr, cg=cg, quant=quant, parts=[p.contiguous().to(dev) for p in cp], res=cr.to(dev), gamma=cg.to(dev),
+                 res_out=torch.empty((t, h), dtype=dtype, device=dev), q=torch.empty((t, h), dtype=torch.uint8, device=dev),
+                 sc=torch.empty((t,), dtype=torch.float32, device=dev), prob=_capi.make_problem(dcode, n, t, h, 1e-5, quant=qm),
+                 stream=torch.cuda.Stream())
+        jobs.append(d)
+    torch.cuda.synchronize()
+    for _ in range(6):
+        for d in jobs:
+            _capi.reduce_rms(d["prob"], [p.data_ptr() for p in d["parts"]], d["res"].data_ptr(), d["res_out"].data_ptr(),
+                             d["gamma"].data_ptr(), q_out=d["q"].data_ptr(), scale_out=d["sc"].data_ptr(),
+                             stream=d["stream"].cuda_stream)
+    torch.cuda.synchronize()
+    for d in jobs:
+        q = d["q"].cpu()
+        got = {"residual_out": d["res_out"].cpu(), "scale": d["sc"].cpu(),
+               "q": q.view(torch.float8_e4m3fn) if d["quant"] == "fp8_token" else q.view(torch.int8)}
+        check_against_oracle(got, eager.reduce_rms(d["cp"], d["cr"], d["cg"], 1e-5, d["quant"]), d["quant"], gamma=d["cg"], eps=1e-5)
