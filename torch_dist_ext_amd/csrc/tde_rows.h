@@ -467,10 +467,9 @@ __global__ void __launch_bounds__(1024 / VPT)
     __attribute__((amdgpu_waves_per_eu(VPT == 1 ? 8 : (VPT == 2 ? 5 : 3)))) row_kernel(const RowArgs a) {
     constexpr int VEC = E::VEC;
     constexpr int NP = (N == 0) ? 1 : N;
-    // Where residual_out is stored.  With 8 partials per row the stores go out together with the row's other
-    // output at the end (one write burst per row: 0.9 % faster on 8 x [2048, 8192] bf16 -> fp8); with fewer
-    // partials storing as soon as the sum is known measures 0.6-1.3 % faster.
-    constexpr bool LATE_RESIDUAL = (N >= 8);
+    // residual_out is stored together with the row's other output at the end, one write burst per row: against storing
+    // it as soon as the sum is known that measures 0.9 % faster on 8 x [2048, 8192] bf16 -> fp8, 0.4 % on 4 x [8192, 7168]
+    // -> fp8 per group, 2.6 % on 2 x [8192, 8192], 7 % on 4 x [512, 7168], and the same within noise elsewhere.
     // Dynamic LDS: the workgroup's squares (one float per element it holds), then 1024 floats of block sums.
     extern __shared__ __attribute__((aligned(16))) float lds_dyn[];
     float *const lds_img = lds_dyn;
@@ -607,7 +606,6 @@ __global__ void __launch_bounds__(1024 / VPT)
 #pragma unroll
             for (int i = 0; i < VEC; ++i) x[i] = s[i] + res[i];
             xraw[j] = E::pack(x);
-            if constexpr (!LATE_RESIDUAL) rsrc_store16(res_out, TDE_OFF(j), xraw[j]);
             E::unpack(xraw[j], x);
             float sq[VEC];
 #pragma unroll
@@ -657,7 +655,7 @@ __global__ void __launch_bounds__(1024 / VPT)
             }
         }
 
-        if constexpr (LATE_RESIDUAL && Q == TDE_QUANT_NONE) {
+        if constexpr (Q == TDE_QUANT_NONE) {
 #pragma unroll
             for (int j = 0; j < VPT; ++j) rsrc_store16(res_out, TDE_OFF(j), xraw[j]);
         }
@@ -693,10 +691,8 @@ __global__ void __launch_bounds__(1024 / VPT)
                 if (row_ok && TDE_T == 0) ((TDE_GLOBAL float *)a.scale_out)[row] = sc;
             }
             const rsrc_t q_out = row_rsrc(a.q_out, row * (int64_t)a.hidden, row_ok ? (uint32_t)a.hidden : 0u);
-            if constexpr (LATE_RESIDUAL) {
 #pragma unroll
-                for (int j = 0; j < VPT; ++j) rsrc_store16(res_out, TDE_OFF(j), xraw[j]);
-            }
+            for (int j = 0; j < VPT; ++j) rsrc_store16(res_out, TDE_OFF(j), xraw[j]);
             // One wavefront-uniform decision for all of the thread's vectors, so the common path carries no per-lane
             // branch: the fast quotient needs every divisor far from the subnormal and overflow ranges.
             bool unsafe = false;
