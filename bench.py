@@ -28,8 +28,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 # (scaled by the plain-copy calibration described there).  They describe the kernels whose sources hash to
 # `sources_sha256`; with any other kernel source the bench line reports traffic as null.
 TRAFFIC = {
-    "sources_sha256": "33a97b13590013d364148f65753593367a8bbcb64abe5f0ec9c19b3956b80228",
-    "bytes": {"c2": 11697330, "c3": 352653695, "c4": 765481471, "c5": 2181192678},
+    "sources_sha256": "744b52e95e0c89bd3e672bd164b8f5d2aa749136cb591e0b2a7ef366d77fc475",
+    "bytes": {"c2": 11694329, "c3": 352653894, "c4": 765469052, "c5": 2181247904},
 }
 
 BENCH_CONFIGS = {

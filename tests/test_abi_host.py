@@ -248,7 +248,7 @@ def test_bench_draws_the_configurations_seeded_inputs():
     (dict(nranks=8, tokens=128, hidden=4096), 1, 512),                               # c2
     (dict(nranks=8, tokens=2048, hidden=8192), 4, 256),                              # c3
     (dict(nranks=4, tokens=8192, hidden=7168), 4, 256),                              # c4
-    (dict(dtype=_capi.F16, nranks=4, tokens=32768, hidden=5120), 1, 640),            # c5, 32768 rows
+    (dict(dtype=_capi.F16, nranks=4, tokens=32768, hidden=5120), 4, 192),            # c5, 32768 rows
     (dict(dtype=_capi.F16, nranks=4, tokens=4096, hidden=5120), 2, 320),             # c5, 4096 rows
     (dict(dtype=_capi.F16, nranks=4, tokens=512, hidden=5120), 1, 640),              # c5, 512 rows
     # the measured boundaries of the choice
@@ -258,7 +258,7 @@ def test_bench_draws_the_configurations_seeded_inputs():
     (dict(nranks=8, tokens=2048, hidden=2048), 4, 64), (dict(nranks=8, tokens=2047, hidden=2048), 1, 256),
     (dict(nranks=4, tokens=32768, hidden=2048), 1, 256),
     (dict(nranks=8, tokens=640, hidden=5120), 2, 320), (dict(nranks=8, tokens=2048, hidden=5120), 1, 640),
-    (dict(nranks=2, tokens=32768, hidden=5120), 2, 320), (dict(nranks=4, tokens=16384, hidden=5120), 1, 640),
+    (dict(nranks=2, tokens=32768, hidden=5120), 2, 320), (dict(nranks=4, tokens=16384, hidden=5120), 4, 192), (dict(nranks=4, tokens=16383, hidden=5120), 2, 320),
 ])
 def test_plan_vectors_per_thread(kw, vpt, threads):
     """The launch geometry tde_plan chooses where the sweeps put a boundary (threads = one row's share)."""

@@ -123,9 +123,12 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     } else if (nvec == 640) {
         // Ten wavefronts per row leave the compute units unevenly filled: from 640 rows up five wavefronts with two
         // vectors each are 10-21 % faster until there are enough rows to even that out (2048 with eight partials,
-        // 16384 with four; with two partials one vector per thread stays 16 % behind at any size).
+        // 16384 with four; with two partials one vector per thread stays 16 % behind at any size).  With four partials
+        // and 16384+ rows all three choices are within 1 %; four vectors per thread is the one whose launches take the
+        // same time from the first on (with one, launches 5 to 50 of a cold run took up to 30 % longer).
         const int64_t even_from = p->nranks >= 8 ? 2048 : (p->nranks == 4 ? 16384 : INT64_MAX);
         if (p->tokens >= 640 && p->tokens < even_from) vpt = 2;
+        else if (p->nranks == 4 && p->tokens >= even_from) vpt = 4;
     }
     if (p->tune_vecs_per_thread != 0) {
         if (p->tune_vecs_per_thread != 1 && p->tune_vecs_per_thread != 2 && p->tune_vecs_per_thread != 4) return TDE_EINVAL;
