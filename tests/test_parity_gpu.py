@@ -207,6 +207,26 @@ def test_rank_order_vector_on_gpu(cuda_device):
     assert torch.all(got["residual_out"].float() == 1.0)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("vpt", [1, 2, 4])
+def test_rank_order_vector_every_geometry(cuda_device, vpt, dtype):
+    """The order-sensitive sum in every accumulation path (vector by vector; rank by rank as the loads arrive with four
+    vectors per thread), four and eight partials: ((((0 + a) + 1) - a) + 1) = 1 only in rank order, with a large enough
+    for a + 1 to round back to a."""
+    # fp16 cannot hold 2^24, but 2^15 + 2^-10 rounds back to 2^15 in the fp32 accumulator just the same
+    big, small = (2.0 ** 24, 1.0) if dtype != torch.float16 else (2.0 ** 15, 2.0 ** -10)
+    hidden = 2048
+    for vals in ([big, small, -big, small], [big, small, -big, small, big, small, -big, small]):
+        n = len(vals)
+        parts = torch.tensor(vals, dtype=dtype).view(n, 1, 1).expand(n, 5, hidden).contiguous()
+        r = torch.zeros((5, hidden), dtype=dtype)
+        g = torch.ones((hidden,), dtype=dtype)
+        want = eager.reduce_rms(parts, r, g, 1e-6, "none")
+        assert torch.all(want["residual_out"].float() == small)
+        got = run_hip(parts, r, g, 1e-6, "none", vecs_per_thread=vpt)
+        assert torch.all(got["residual_out"].float() == small), (vpt, n)
+
+
 def test_sum_of_ones_row_reduction_all_wave_counts(cuda_device):
     # mean(x^2) of a row of ones is exactly 1 for every hidden: checks the 64-lane + LDS reduction tree
     for hidden in (8, 64, 1016, 1024, 5120, 7168, 8192):
