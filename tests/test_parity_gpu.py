@@ -456,13 +456,15 @@ def test_hip_graph_replays_match_eager(cuda_device, algo):
 
 @pytest.mark.parametrize("quant", ["none", "fp8_token", "fp8_group", "int8_token"])
 @pytest.mark.parametrize("dtype,hidden", [(torch.float16, 8192), (torch.float32, 4096), (torch.bfloat16, 7168), (torch.float32, 3584)])
-def test_long_rows_every_dtype(cuda_device, dtype, hidden, quant):
+@pytest.mark.parametrize("n", [2, 4, 8])
+def test_long_rows_every_dtype(cuda_device, dtype, hidden, quant, n):
     """Rows of 896..1024 vectors take the 4-vectors-per-thread kernels once there are many rows; cover them
-    for every dtype and mode (forced here, the input has few rows)."""
-    p, r, g = eager.make_inputs(4, 19, hidden, dtype, 1.0, seed=hidden + 3)
+    for every dtype, mode and number of partials (forced here, the input has few rows): with four and eight
+    partials these are the kernels that sum rank by rank while the loads arrive."""
+    p, r, g = eager.make_inputs(n, 19, hidden, dtype, 1.0, seed=hidden + 3 + n)
     code = {torch.float16: _capi.F16, torch.float32: _capi.F32, torch.bfloat16: _capi.BF16}[dtype]
-    assert _capi.plan(_capi.make_problem(code, 4, 4096, hidden, 1e-6)).vecs_per_thread == 4
-    assert _capi.plan(_capi.make_problem(code, 4, 19, hidden, 1e-6)).vecs_per_thread == 1
+    assert _capi.plan(_capi.make_problem(code, n, 4096, hidden, 1e-6)).vecs_per_thread == 4
+    assert _capi.plan(_capi.make_problem(code, n, 19, hidden, 1e-6)).vecs_per_thread == 1
     _case("long-rows", p, r, g, 1e-6, quant, vecs_per_thread=4)
 
 
