@@ -12,7 +12,8 @@ namespace tde {
 
 // CODE_BYTES: bytes of quantized output per 16-byte input vector (0 none, 4 for fp32 rows, 8 for 2-byte rows).
 template <int N, int VPT, int CODE_BYTES, bool WN>
-__global__ void __launch_bounds__(1024 / VPT) traffic_kernel(const RowArgs a, uint32_t row_bytes) {
+__global__ void __launch_bounds__(1024 / VPT)
+    __attribute__((amdgpu_waves_per_eu(VPT == 1 ? 8 : (VPT == 2 ? 5 : 3)))) traffic_kernel(const RowArgs a, uint32_t row_bytes) {
     constexpr int NP = (N == 0) ? 1 : N;
     const int tid = threadIdx.x;
     const int tpr = a.threads_per_row;
@@ -86,8 +87,11 @@ __global__ void __launch_bounds__(1024 / VPT) traffic_kernel(const RowArgs a, ui
 template <int N, int VPT>
 hipError_t launch_traffic_nv(int code_bytes, bool wn, const RowArgs &a, const Geometry &g, uint32_t row_bytes, hipStream_t s) {
     const dim3 grid((unsigned)g.grid), block((unsigned)g.block_threads);
+    // The LDS the row kernel of this geometry allocates (never touched here) and its wavefronts-per-SIMD bound: the
+    // skeleton then fills a compute unit with as many workgroups as the kernel does.
+    const size_t lds = sumsq_lds_bytes(g.block_threads, VPT, g.vec_elems);
 #define TDE_TRAFFIC(CB, WNB)                                                                   \
-    hipLaunchKernelGGL((traffic_kernel<N, VPT, CB, WNB>), grid, block, 0, s, a, row_bytes); \
+    hipLaunchKernelGGL((traffic_kernel<N, VPT, CB, WNB>), grid, block, lds, s, a, row_bytes); \
     return hipGetLastError();
     if (code_bytes == 0) { TDE_TRAFFIC(0, true) }
     if (code_bytes == 8) { if (wn) { TDE_TRAFFIC(8, true) } else { TDE_TRAFFIC(8, false) } }
