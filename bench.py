@@ -28,8 +28,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 # (scaled by the plain-copy calibration described there).  They describe the kernels whose sources hash to
 # `sources_sha256`; with any other kernel source the bench line reports traffic as null.
 TRAFFIC = {
-    "sources_sha256": "81f91c4dd92ee4b77f45f60ee7576739d387c5c573905c98f2375c46591e42e1",
-    "bytes": {"c2": 11694426, "c3": 352654227, "c4": 765467105, "c5": 2181233650},
+    "sources_sha256": "254461f538631410e2c325304288d663c129ea28e95510534876a939cb47bade",
+    "bytes": {"c2": 11694499, "c3": 352653711, "c4": 765468995, "c5": 2181269391},
 }
 
 BENCH_CONFIGS = {
