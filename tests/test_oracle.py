@@ -209,6 +209,36 @@ def test_c_restatement_in_torch_sum_order_is_bit_identical_to_eager(dtype, code,
         assert np.array_equal(c["q"], want["q"].view(torch.uint8).numpy())
 
 
+def test_c_restatement_against_eager_over_random_shapes():
+    """The two statements of the oracle (torch eager and the integer C restatement in torch's summation order) agree
+    bit for bit over a seeded sweep of shapes, element types, numbers of partials and quant modes, including row
+    lengths with left-over vectors, left-over scalars and short last blocks."""
+    rng = np.random.default_rng(20240611)
+    types = [(torch.bfloat16, cport.BF16, 8), (torch.float16, cport.F16, 8), (torch.float32, cport.F32, 4)]
+    for case in range(60):
+        dtype, code, vec = types[int(rng.integers(0, 3))]
+        n = int(rng.choice([2, 4, 8]))
+        tokens = int(rng.integers(1, 12))
+        hidden = vec * int(rng.integers(1, 700 if vec == 8 else 900))
+        quant = ["none", "fp8_token", "int8_token", "fp8_group"][int(rng.integers(0, 4))]
+        if quant == "fp8_group":
+            hidden = 128 * max(1, hidden // 128)
+        sigma = float(rng.choice([0.01, 1.0, 30.0]))
+        p, r, g = eager.make_inputs(n, tokens, hidden, dtype, sigma, seed=1000 + case)
+        want = eager.reduce_rms(p, r, g, 1e-6, quant)
+        if dtype == torch.float32:
+            conv, back = (lambda t: t.numpy()), (lambda a: torch.from_numpy(a))
+        else:
+            conv, back = _bits16, (lambda a, dtype=dtype: _from_bits16(a, dtype))
+        c = cport.reduce_rms(code, [conv(p[i]) for i in range(n)], conv(r), conv(g), 1e-6, quant=quant, sumsq_mode=cport.SUMSQ_TORCH)
+        label = (case, dtype, n, tokens, hidden, quant, sigma)
+        assert bits_equal(back(c["residual_out"]), want["residual_out"]), label
+        assert bits_equal(back(c["norm_out"]), want["norm_out"]), label
+        if quant != "none":
+            assert np.array_equal(c["scale"].reshape(-1).view(np.uint32), want["scale"].numpy().reshape(-1).view(np.uint32)), label
+            assert np.array_equal(c["q"].reshape(-1).view(np.uint8), want["q"].view(torch.uint8).numpy().reshape(-1)), label
+
+
 def test_library_rms_norm_cross_check():
     p, r, g = eager.make_inputs(2, 8, 512, torch.bfloat16, 1.0, seed=9)
     x = eager.reduce_residual(p, r)
