@@ -24,9 +24,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 
-# HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs summarized under profiles/
-# (scaled by the plain-copy calibration described there).  They describe the kernels whose sources hash to
-# `sources_sha256`; with any other kernel source the bench line reports traffic as null.
+# HBM bytes per launch, measured with two rocprofv3 counter runs of this script per configuration (--pmc FETCH_SIZE,
+# then --pmc WRITE_SIZE; KiB per dispatch of the row kernel), each scaled by what the same counter reads for the three
+# 256 MiB calibration copies this script dispatches before its warm-up (FETCH_SIZE reads half the bytes on this part).
+# They describe the kernels whose sources hash to `sources_sha256`; with any other kernel source the bench line reports
+# traffic as null.
 TRAFFIC = {
     "sources_sha256": "254461f538631410e2c325304288d663c129ea28e95510534876a939cb47bade",
     "bytes": {"c2": 11694499, "c3": 352653711, "c4": 765468995, "c5": 2181269391},
