@@ -30,8 +30,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 # They describe the kernels whose sources hash to `sources_sha256`; with any other kernel source the bench line reports
 # traffic as null.
 TRAFFIC = {
-    "sources_sha256": "254461f538631410e2c325304288d663c129ea28e95510534876a939cb47bade",
-    "bytes": {"c2": 11694499, "c3": 352653711, "c4": 765468995, "c5": 2181269391},
+    "sources_sha256": "68b2755a74d39b1e1eeebda92ddc4fe883bf74510a247b8982db8c7705f5b58a",
+    "bytes": {"c2": 11695533, "c3": 352654622, "c4": 765470798, "c5": 2181272392},
 }
 
 BENCH_CONFIGS = {
@@ -134,6 +134,8 @@ def main():
     ap.add_argument("--sets", type=int, default=0, help="distinct input sets to rotate over (0 = enough for > 1 GiB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--algo", default="auto", choices=["auto", "fused", "staged", "staged_owned"])
+    ap.add_argument("--workgroups-per-cu", type=int, default=0,
+                    help="limit on resident workgroups per compute unit: 0 = the library's choice, -1 = none, 1..8 = forced")
     ap.add_argument("--print-source-hash", action="store_true", help="print the kernel-source hash and exit")
     args = ap.parse_args()
     if args.print_source_hash:
@@ -159,7 +161,7 @@ def main():
     algo = {"auto": _capi.ALGO_AUTO, "fused": _capi.ALGO_FUSED, "staged": _capi.ALGO_STAGED,
             "staged_owned": _capi.ALGO_STAGED_OWNED}[args.algo]
     dcode = {"bf16": _capi.BF16, "f16": _capi.F16, "f32": _capi.F32}[dt]
-    prob = _capi.make_problem(dcode, N, T, H, eps, quant=qm, algo=algo, write_norm=0)
+    prob = _capi.make_problem(dcode, N, T, H, eps, quant=qm, algo=algo, write_norm=0, workgroups_per_cu=args.workgroups_per_cu)
     plan = _capi.plan(prob)
     bytes_per_launch = plan.algorithmic_bytes
     # Enough distinct sets that a buffer is touched again only after > 4 GiB of other inputs AND > 1 GiB of other
@@ -297,7 +299,7 @@ def main():
                        {"staged": " (two launches through a stage buffer)",
                         "staged_owned": " (two launches; stage A over this rank's T/N rows only)"}.get(args.algo, "")),
                    "storage_dtype": dt, "output": quant, "algo": args.algo, "input_sets": nsets, "block_threads": plan.block_threads,
-                   "grid_blocks": plan.grid_blocks, "algorithmic_bytes": bytes_per_launch},
+                   "workgroups_per_cu": plan.workgroups_per_cu, "grid_blocks": plan.grid_blocks, "algorithmic_bytes": bytes_per_launch},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel_avg_us": avg_ms * 1e3,

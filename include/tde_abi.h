@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define TDE_ABI_VERSION 2
+#define TDE_ABI_VERSION 3
 #define TDE_MAX_RANKS 16 /* array bound, as MAX_RANKS in src/ops/all_reduce_fusion.h:8 */
 #define TDE_QUANT_GROUP 128
 #define TDE_STATIC_STAGE_BYTES (32 << 20) /* stage held inside the library for tde_reduce_rms_static_stage */
@@ -98,6 +98,9 @@ typedef struct tde_problem {
     int32_t tune_vecs_per_thread; /* 1, 2 or 4 16-byte vectors per thread per row (other non-zero values: TDE_EINVAL) */
     int32_t tune_rows_per_block;  /* rows side by side in one workgroup; ignored where it would exceed the
                                      kernel's launch bound of 1024 / vecs_per_thread threads */
+    int32_t tune_workgroups_per_cu; /* at most this many workgroups resident per compute unit (1..8; enforced by
+                                       padding the launch's dynamic LDS); -1 = no limit; other values: TDE_EINVAL */
+    int32_t reserved;               /* must be 0 */
 } tde_problem;
 
 typedef struct tde_buffers {
@@ -128,6 +131,8 @@ typedef struct tde_plan_out {
     int32_t grid_blocks;     /* workgroups launched for the row kernel */
     int32_t xcd_chunk;       /* row groups each XCD takes in a row: workgroup b of every 8*xcd_chunk takes row group
                                 (b % 8) * xcd_chunk + b / 8 of that span (1 = launch order) */
+    int32_t workgroups_per_cu; /* limit on resident workgroups per compute unit the launch enforces (0 = none) */
+    int32_t lds_bytes;         /* dynamic LDS per workgroup of the row kernel's launch, padding included */
     int64_t algorithmic_bytes; /* (N+1)*T*H*e + H*e + T*H*e + OUT, OUT as documented for the quant mode */
     int64_t scale_elems;       /* number of fp32 scales written */
 } tde_plan_out;

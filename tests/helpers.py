@@ -38,13 +38,14 @@ def bits_equal(a: torch.Tensor, b: torch.Tensor) -> bool:
 
 
 def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, write_norm=None, use_table=False,
-            rank=0, device="cuda:0", static_scale=0.0, stage_init=None, calls=None, vecs_per_thread=0, rows_per_block=0):
+            rank=0, device="cuda:0", static_scale=0.0, stage_init=None, calls=None, vecs_per_thread=0, rows_per_block=0,
+            workgroups_per_cu=0):
     """Run the HIP path through the C ABI (tde_reduce_rms) on CPU inputs; returns CPU outputs.
     parts: [N,T,H] tensor or list of N [T,H] tensors.  stage_init: [T,H] initial content of the stage
     buffer (staged algorithms); the stage is then returned as out["stage"].  calls: sequence of
     (phases, rank) issued in order on the same buffers instead of the one tde_reduce_rms call, e.g.
-    [(("reduce",), 0), (("reduce",), 1), (("norm",), 0)].  vecs_per_thread / rows_per_block: the per-call
-    launch-geometry overrides of tde_problem (0 = automatic)."""
+    [(("reduce",), 0), (("reduce",), 1), (("norm",), 0)].  vecs_per_thread / rows_per_block / workgroups_per_cu: the
+    per-call launch-geometry overrides of tde_problem (0 = automatic)."""
     dev = torch.device(device)
     n = len(parts)
     T, H = residual.shape
@@ -85,7 +86,7 @@ def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, wri
     for phases, call_rank in (calls or [(("reduce", "norm"), rank)]):
         prob = _capi.make_problem(DTYPE_CODE[dtype], n, T, H, eps, quant=qm, algo=algo, write_norm=int(bool(write_norm)),
                                   rank=call_rank, static_scale=static_scale, vecs_per_thread=vecs_per_thread,
-                                  rows_per_block=rows_per_block)
+                                  rows_per_block=rows_per_block, workgroups_per_cu=workgroups_per_cu)
         _capi.reduce_rms(prob, ptrs, d_res.data_ptr(), d_res_out.data_ptr(), d_gamma.data_ptr(),
                          norm_out=d_norm.data_ptr() if d_norm is not None else None,
                          q_out=d_q.data_ptr() if d_q is not None else None,

@@ -26,13 +26,13 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), name
     assert sorted(_capi.EXPORTS) == declared
-    assert _capi.load().tde_abi_version() == 2
+    assert _capi.load().tde_abi_version() == _capi.ABI_VERSION == 3
 
 
 def test_struct_layouts_match_header():
-    assert ctypes.sizeof(_capi.Problem) == 56
+    assert ctypes.sizeof(_capi.Problem) == 64
     assert ctypes.sizeof(_capi.Buffers) == (16 + 8) * 8
-    assert ctypes.sizeof(_capi.PlanOut) == 48
+    assert ctypes.sizeof(_capi.PlanOut) == 56
 
 
 def _plan(**kw):
@@ -264,3 +264,45 @@ def test_plan_vectors_per_thread(kw, vpt, threads):
     """The launch geometry tde_plan chooses where the sweeps put a boundary (threads = one row's share)."""
     p = _plan(**kw)
     assert (p.vecs_per_thread, p.block_threads // p.rows_per_block) == (vpt, threads)
+
+
+@pytest.mark.parametrize("kw,limit,lds", [
+    # fewer than 6144 workgroups, two partials, the staged algorithms and doubles: no limit, LDS = what the reduction needs
+    (dict(nranks=8, tokens=2048, hidden=8192), 0, (256 * 4 * 8 + 1024) * 4),
+    (dict(nranks=8, tokens=6143, hidden=8192), 0, (256 * 4 * 8 + 1024) * 4),
+    (dict(nranks=2, tokens=32768, hidden=8192), 0, (256 * 4 * 8 + 1024) * 4),
+    (dict(nranks=8, tokens=32768, hidden=8192, algo=_capi.ALGO_STAGED), 0, (256 * 4 * 8 + 1024) * 4),
+    # long launches: about 128 KiB of loads in flight per CU, never fewer than two workgroups or eight wavefronts
+    (dict(nranks=8, tokens=6144, hidden=8192), 2, 80896),                                    # 144 KiB per workgroup
+    (dict(nranks=4, tokens=32768, hidden=8192), 2, 80896),                                   # 80 KiB per workgroup
+    (dict(nranks=4, tokens=32768, hidden=5120, dtype=_capi.F16, quant=_capi.QUANT_INT8_TOKEN), 3, 53504),  # 3 wavefronts each
+    (dict(nranks=4, tokens=12288, hidden=7168, quant=_capi.QUANT_FP8_GROUP), 3, 53504),     # twelve wavefronts for group scales
+    (dict(nranks=4, tokens=12288, hidden=7168, quant=_capi.QUANT_FP8_TOKEN), 2, 80896),
+    (dict(nranks=4, tokens=12287, hidden=7168, quant=_capi.QUANT_FP8_TOKEN), 0, (256 * 4 * 8 + 1024) * 4),  # four partials: from 12288
+    (dict(nranks=8, tokens=32768, hidden=1024), 4, 39936),                                   # 2 rows x 18 KiB per workgroup
+    (dict(nranks=4, tokens=32768, hidden=2048), 6, 26112),
+    # the per-call override
+    (dict(nranks=8, tokens=16, hidden=1024, workgroups_per_cu=1), 1, 162816),
+    (dict(nranks=8, tokens=16, hidden=1024, workgroups_per_cu=8), 8, 19456),
+    (dict(nranks=8, tokens=32768, hidden=8192, workgroups_per_cu=-1), 0, (256 * 4 * 8 + 1024) * 4),
+])
+def test_plan_workgroups_per_cu(kw, limit, lds):
+    """The limit on resident workgroups per compute unit and the dynamic LDS that enforces it."""
+    p = _plan(**kw)
+    assert (p.workgroups_per_cu, p.lds_bytes) == (limit, lds)
+    if limit:   # `limit` workgroups of this LDS (plus the kernels' 64 static bytes) fit 160 KiB, one more does not
+        assert limit * (lds + 64) <= 160 * 1024 < (limit + 1) * (lds + 64)
+
+
+@pytest.mark.parametrize("kw", [dict(workgroups_per_cu=9), dict(workgroups_per_cu=-2)])
+def test_plan_rejects_workgroup_limits_out_of_range(kw):
+    with pytest.raises(_capi.TdeError) as err:
+        _plan(**kw)
+    assert err.value.status == _capi.EINVAL
+
+
+def test_plan_rejects_nonzero_reserved_field():
+    prob = _capi.make_problem(_capi.BF16, 8, 16, 1024, 1e-6)
+    prob.reserved = 1
+    assert _capi.load().tde_plan(ctypes.byref(prob), ctypes.byref(_capi.PlanOut())) == _capi.EINVAL
+

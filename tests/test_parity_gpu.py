@@ -253,6 +253,52 @@ def test_every_launch_geometry_agrees(cuda_device, vpt, hidden, rows_per_block):
         assert bits_equal(base[key], other[key]), key
 
 
+@pytest.mark.parametrize("limit", [1, 2, 3, 8])
+@pytest.mark.parametrize("n,hidden,dtype,quant", [(8, 8192, torch.bfloat16, "fp8_token"), (4, 7168, torch.bfloat16, "fp8_group"),
+                                                  (4, 5120, torch.float16, "int8_token"), (2, 1024, torch.float32, "none")])
+def test_every_workgroup_limit_agrees(cuda_device, limit, n, hidden, dtype, quant):
+    """A forced limit on resident workgroups per CU pads the launch's dynamic LDS (beyond 64 KiB for limits 1 and 2,
+    which needs the kernel's LDS ceiling raised first) and changes nothing else."""
+    p, r, g = eager.make_inputs(n, 53, hidden, dtype, 0.5, seed=91)
+    base = run_hip(p, r, g, 1e-5, quant, workgroups_per_cu=-1)
+    other = run_hip(p, r, g, 1e-5, quant, workgroups_per_cu=limit)
+    check_against_oracle(other, eager.reduce_rms(p, r, g, 1e-5, quant), quant, gamma=g, eps=1e-5)
+    for key in base:
+        assert bits_equal(base[key], other[key]), key
+
+
+def test_long_launch_with_automatic_workgroup_limit(cuda_device):
+    """6144 rows of 8 partials: the plan limits the launch to two workgroups per CU (79 KiB of dynamic LDS each).
+    Same bits as the unlimited launch, on the device."""
+    dev = cuda_device
+    n, t, h = 8, 6144, 5120
+    prob = _capi.make_problem(_capi.BF16, n, t, h, 1e-5, quant=_capi.QUANT_FP8_TOKEN)
+    plan = _capi.plan(prob)
+    assert plan.workgroups_per_cu == 2 and plan.lds_bytes > 64 * 1024
+    gen = torch.Generator(device=dev).manual_seed(17)
+    parts = [(torch.randn((t, h), generator=gen, device=dev) * 0.5).to(torch.bfloat16) for _ in range(n)]
+    res = torch.randn((t, h), generator=gen, device=dev).to(torch.bfloat16)
+    gamma = (torch.rand((h,), generator=gen, device=dev) + 0.5).to(torch.bfloat16)
+    outs = []
+    for limit in (0, -1):
+        res_out = torch.full_like(res, float("nan"))
+        q = torch.full((t, h), 0xFF, dtype=torch.uint8, device=dev)
+        sc = torch.full((t,), float("nan"), dtype=torch.float32, device=dev)
+        call = _capi.make_problem(_capi.BF16, n, t, h, 1e-5, quant=_capi.QUANT_FP8_TOKEN, workgroups_per_cu=limit)
+        _capi.reduce_rms(call, [p.data_ptr() for p in parts], res.data_ptr(), res_out.data_ptr(), gamma.data_ptr(),
+                         q_out=q.data_ptr(), scale_out=sc.data_ptr(), stream=torch.cuda.current_stream(dev).cuda_stream)
+        torch.cuda.synchronize(dev)
+        outs.append((res_out, q, sc))
+    for a, b in zip(*outs):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+    acc = torch.zeros((t, h), device=dev)
+    for p in parts:
+        acc = acc + p.float()
+    x = (acc.to(torch.bfloat16).float() + res.float()).to(torch.bfloat16)
+    assert torch.equal(outs[0][0].view(torch.int16), x.view(torch.int16))
+    assert torch.all(outs[0][1].view(torch.float8_e4m3fn).float().abs().amax(-1) == 448.0)
+
+
 def test_full_size_c3_properties(cuda_device):
     """Configuration c3 at full size on the device only (the CPU oracle is not run at this size here):
     size-independent properties of the outputs."""

@@ -17,6 +17,8 @@ QUANT_NONE, QUANT_FP8_TOKEN, QUANT_FP8_GROUP, QUANT_INT8_TOKEN, QUANT_FP8_STATIC
 ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, ALGO_STAGED_OWNED = 0, 1, 2, 3
 
 # Every symbol include/tde_abi.h declares.
+ABI_VERSION = 3   # TDE_ABI_VERSION of include/tde_abi.h
+
 EXPORTS = (
     "tde_abi_version", "tde_status_string", "tde_last_hip_error", "tde_plan", "tde_reduce_rms", "tde_stage_reduce", "tde_stage_norm",
     "tde_reduce_rms_static_stage",
@@ -32,6 +34,7 @@ class Problem(ctypes.Structure):
         ("algo", ctypes.c_int32), ("write_norm", ctypes.c_int32), ("tokens", ctypes.c_int64), ("hidden", ctypes.c_int64),
         ("eps", ctypes.c_float), ("static_scale", ctypes.c_float),
         ("tune_vecs_per_thread", ctypes.c_int32), ("tune_rows_per_block", ctypes.c_int32),
+        ("tune_workgroups_per_cu", ctypes.c_int32), ("reserved", ctypes.c_int32),
     ]
 
 
@@ -47,7 +50,8 @@ class PlanOut(ctypes.Structure):
     _fields_ = [
         ("algo", ctypes.c_int32), ("reference_algo", ctypes.c_int32), ("vec_elems", ctypes.c_int32),
         ("block_threads", ctypes.c_int32), ("vecs_per_thread", ctypes.c_int32), ("rows_per_block", ctypes.c_int32),
-        ("grid_blocks", ctypes.c_int32), ("xcd_chunk", ctypes.c_int32), ("algorithmic_bytes", ctypes.c_int64),
+        ("grid_blocks", ctypes.c_int32), ("xcd_chunk", ctypes.c_int32), ("workgroups_per_cu", ctypes.c_int32),
+        ("lds_bytes", ctypes.c_int32), ("algorithmic_bytes", ctypes.c_int64),
         ("scale_elems", ctypes.c_int64),
     ]
 
@@ -77,6 +81,9 @@ def load():
         raise ImportError("%s not built; run `python torch_dist_ext_amd/_build.py`" % LIB_PATH)
     lib = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
     lib.tde_abi_version.restype = ctypes.c_int
+    if lib.tde_abi_version() != ABI_VERSION:   # the structures below mirror one version of include/tde_abi.h
+        raise ImportError("%s has ABI version %d, this module is written for %d; rebuild it"
+                          % (LIB_PATH, lib.tde_abi_version(), ABI_VERSION))
     lib.tde_status_string.restype = ctypes.c_char_p
     lib.tde_status_string.argtypes = [ctypes.c_int]
     lib.tde_last_hip_error.restype = ctypes.c_int
@@ -128,10 +135,11 @@ def check(status):
 
 
 def make_problem(dtype, nranks, tokens, hidden, eps, quant=QUANT_NONE, algo=ALGO_AUTO, write_norm=0, rank=0,
-                 static_scale=0.0, vecs_per_thread=0, rows_per_block=0):
+                 static_scale=0.0, vecs_per_thread=0, rows_per_block=0, workgroups_per_cu=0):
     return Problem(dtype=dtype, nranks=nranks, rank=rank, quant=quant, algo=algo, write_norm=int(write_norm),
                    tokens=tokens, hidden=hidden, eps=eps, static_scale=static_scale,
-                   tune_vecs_per_thread=vecs_per_thread, tune_rows_per_block=rows_per_block)
+                   tune_vecs_per_thread=vecs_per_thread, tune_rows_per_block=rows_per_block,
+                   tune_workgroups_per_cu=workgroups_per_cu)
 
 
 def plan(problem):

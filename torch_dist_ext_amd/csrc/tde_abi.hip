@@ -2,6 +2,8 @@
 // workspace.  Declarations and the reference interfaces they replace are in include/tde_abi.h.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include <cstdint>
 #include <cstring>
 #include <mutex>
@@ -59,6 +61,9 @@ int static_stage_ptr(void **out) {
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 constexpr int kMaxBlock = 1024;
+constexpr int64_t kLoadsInFlightPerCu = 128 * 1024; // target for the limit on resident workgroups (see validate)
+// launches with fewer workgroups are not limited (8 partials; twice as many with 4, whose launches are half as long)
+constexpr int64_t kLimitWorkgroupsFromGrid = 6144;
 constexpr int kDefaultComputeUnits = 256; // MI355X; used when no device can be asked (planning on a host without one)
 
 // Compute units of the current device, asked once per device.
@@ -135,6 +140,7 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
         vpt = p->tune_vecs_per_thread;
     }
     if (p->tune_rows_per_block < 0) return TDE_EINVAL;
+    if (p->tune_workgroups_per_cu < -1 || p->tune_workgroups_per_cu > 8 || p->reserved != 0) return TDE_EINVAL;
     if (p->dtype == TDE_F64) vpt = 1;
     const int64_t lanes = (nvec + vpt - 1) / vpt;
     const int tpr = (int)((lanes + 63) / 64 * 64);
@@ -148,7 +154,32 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     const int64_t grid = (p->tokens + rpb - 1) / rpb; // one workgroup per group of rows, no loop
     if (grid > 0x7fffffff) return TDE_ESHAPE;
 
+    // Resident workgroups per compute unit.  Left alone, a CU takes as many workgroups as its registers and LDS hold
+    // (3-6 here), each with all of its rows' loads in flight.  On MI355X long launches run fastest with 120-160 KiB
+    // of loads in flight per CU: more costs 1-8 % from 8192 rows up with 4 or 8 partials (32768 x 8192: 7.5 % with
+    // 4 partials, 4.5 % with 8; 16384 rows: 1-3 %; 8192 rows with 8 partials: 1 %), fewer than two workgroups or
+    // eight wavefronts per CU leave the arithmetic of one row uncovered by the loads of another.  Short launches (a
+    // few generations of workgroups) gain nothing and can lose 1-3 %, and with 2 partials no limit helps.
+    int wgs_per_cu = 0;
+    const bool staged = p->algo == TDE_ALGO_STAGED || p->algo == TDE_ALGO_STAGED_OWNED; // its row kernel reads 2 streams
+    if (p->dtype != TDE_F64 && !staged && p->nranks >= 4 && grid >= kLimitWorkgroupsFromGrid * (p->nranks >= 8 ? 1 : 2)) {
+        const int64_t per_wg = (int64_t)rpb * (p->nranks + 1) * nvec * 16; // bytes of loads one workgroup keeps in flight
+        const int waves = tpr * rpb / 64;
+        // per-group scales are the heaviest arithmetic per row and four partials the shortest loads to cover it
+        const int need_waves = (p->quant == TDE_QUANT_FP8_GROUP && p->nranks <= 4) ? 12 : 8;
+        const int at_least = std::max(2, (need_waves + waves - 1) / waves);
+        wgs_per_cu = (int)std::min<int64_t>(8, std::max<int64_t>(at_least, (kLoadsInFlightPerCu + per_wg / 2) / per_wg));
+    }
+    if (p->tune_workgroups_per_cu != 0 && p->dtype != TDE_F64) wgs_per_cu = p->tune_workgroups_per_cu < 0 ? 0 : p->tune_workgroups_per_cu;
+
     if (geo) {
+        geo->wgs_per_cu = wgs_per_cu;
+        geo->lds_bytes = 0;
+        if (p->dtype != TDE_F64) {
+            size_t lds = tde::sumsq_lds_bytes(tpr * rpb, vpt, vec);
+            if (wgs_per_cu > 0) lds = std::max(lds, tde::lds_bytes_for_workgroups_per_cu(wgs_per_cu));
+            geo->lds_bytes = (int)lds;
+        }
         geo->vec_elems = vec;
         geo->nvec = (int)nvec;
         geo->vpt = vpt;
@@ -320,6 +351,8 @@ int tde_plan(const tde_problem *problem, tde_plan_out *plan) {
     plan->rows_per_block = g.rows_per_block;
     plan->grid_blocks = (int32_t)g.grid;
     plan->xcd_chunk = g.xcd_chunk;
+    plan->workgroups_per_cu = g.wgs_per_cu;
+    plan->lds_bytes = g.lds_bytes;
     plan->algorithmic_bytes = algorithmic_bytes(problem, &plan->scale_elems);
     return TDE_OK;
 }

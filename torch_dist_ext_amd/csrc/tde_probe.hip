@@ -87,10 +87,14 @@ __global__ void __launch_bounds__(1024 / VPT)
 template <int N, int VPT>
 hipError_t launch_traffic_nv(int code_bytes, bool wn, const RowArgs &a, const Geometry &g, uint32_t row_bytes, hipStream_t s) {
     const dim3 grid((unsigned)g.grid), block((unsigned)g.block_threads);
-    // The LDS the row kernel of this geometry allocates (never touched here) and its wavefronts-per-SIMD bound: the
-    // skeleton then fills a compute unit with as many workgroups as the kernel does.
-    const size_t lds = sumsq_lds_bytes(g.block_threads, VPT, g.vec_elems);
+    // The LDS the row kernel of this geometry allocates (never touched here), padding included, and its
+    // wavefronts-per-SIMD bound: the skeleton then fills a compute unit with as many workgroups as the kernel does.
+    const size_t lds = (size_t)g.lds_bytes;
 #define TDE_TRAFFIC(CB, WNB)                                                                   \
+    if (lds > kDefaultMaxDynamicLds) {                                                         \
+        const hipError_t e = allow_large_lds<traffic_kernel<N, VPT, CB, WNB>>();               \
+        if (e != hipSuccess) return e;                                                         \
+    }                                                                                          \
     hipLaunchKernelGGL((traffic_kernel<N, VPT, CB, WNB>), grid, block, lds, s, a, row_bytes); \
     return hipGetLastError();
     if (code_bytes == 0) { TDE_TRAFFIC(0, true) }

@@ -21,6 +21,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "tde_abi.h"
 
 namespace tde {
@@ -199,6 +201,30 @@ __device__ __forceinline__ float quad_bcast(float v) {
 // Dynamic LDS a kernel that calls sumsq_torch_order needs.
 inline size_t sumsq_lds_bytes(int block_threads, int vpt, int vec_floats) {
     return ((size_t)block_threads * vpt * vec_floats + 1024) * sizeof(float);
+}
+
+// A compute unit of gfx950 has 160 KiB of LDS; a workgroup that asks for this much dynamic LDS (the kernels' 64
+// static bytes and the allocation granule fit in the slack) shares its CU with at most `wgs` - 1 others.
+constexpr size_t kLdsPerCu = 160 * 1024;
+constexpr size_t kDefaultMaxDynamicLds = 64 * 1024; // what a kernel may ask for without raising its attribute
+inline size_t lds_bytes_for_workgroups_per_cu(int wgs) { return (kLdsPerCu / (size_t)wgs - 1024) & ~(size_t)255; }
+
+// Raises KERNEL's dynamic-LDS ceiling to (nearly) the whole CU, once per device (a launch asking for more than 64 KiB
+// fails otherwise).  Not a stream operation; the first launch of a kernel on a device that needs it pays for it.
+template <auto KERNEL>
+hipError_t allow_large_lds() {
+    static std::atomic<uint64_t> done{0}; // bit d: set on device d
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const uint64_t bit = (dev >= 0 && dev < 64) ? (uint64_t{1} << dev) : 0;
+    if (bit != 0 && (done.load(std::memory_order_acquire) & bit)) return hipSuccess;
+    // the most a launch here asks for; the kernel's static LDS must still fit beside it
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(KERNEL), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds_bytes_for_workgroups_per_cu(1));
+    if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+    else (void)hipGetLastError(); // reported through the return value, not left behind for the next call
+    return e;
 }
 
 // Returns `v`, but only once `after` exists: index arithmetic built on the result cannot be hoisted above the
@@ -815,6 +841,8 @@ __global__ void __launch_bounds__(256) reduce_kernel(const RowArgs a, const Redu
 // Host-side launch geometry shared by tde_plan and the launchers.
 // ---------------------------------------------------------------------------------------------
 struct Geometry {
+    int wgs_per_cu; // limit on resident workgroups per compute unit (0 = none), enforced through lds_bytes
+    int lds_bytes;  // dynamic LDS of the row kernel's launch
     int vec_elems;
     int nvec;
     int vpt;
@@ -844,8 +872,12 @@ hipError_t launch_traffic(int n, int vpt, int code_bytes, bool wn, const RowArgs
 template <class E, int N, int VPT>
 hipError_t launch_rows_nv(int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s) {
     const dim3 grid((unsigned)g.grid), block((unsigned)g.block_threads);
-    const size_t lds = sumsq_lds_bytes(g.block_threads, VPT, E::VEC);
+    const size_t lds = (size_t)g.lds_bytes; // sumsq_lds_bytes of this geometry, padded where the launch limits workgroups per CU
 #define TDE_LAUNCH(QM, WNB)                                                         \
+    if (lds > kDefaultMaxDynamicLds) {                                              \
+        const hipError_t e = allow_large_lds<row_kernel<E, N, VPT, QM, WNB>>();     \
+        if (e != hipSuccess) return e;                                              \
+    }                                                                               \
     hipLaunchKernelGGL((row_kernel<E, N, VPT, QM, WNB>), grid, block, lds, s, a); \
     return hipGetLastError();
     switch (q) {
