@@ -239,6 +239,8 @@ def main():
     # (back-to-back launches on one stream; the gap between them is part of it).
     ev0 = torch.cuda.Event(enable_timing=True)
     ev1 = torch.cuda.Event(enable_timing=True)
+    ev0.record(stream)      # torch creates the HIP event at its first record: not inside the timed region
+    ev1.record(stream)
     torch.cuda.synchronize(dev)
     t0 = time.perf_counter()
     ev0.record(stream)
