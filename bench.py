@@ -30,8 +30,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 # They describe the kernels whose sources hash to `sources_sha256`; with any other kernel source the bench line reports
 # traffic as null.
 TRAFFIC = {
-    "sources_sha256": "68b2755a74d39b1e1eeebda92ddc4fe883bf74510a247b8982db8c7705f5b58a",
-    "bytes": {"c2": 11695533, "c3": 352654622, "c4": 765470798, "c5": 2181272392},
+    "sources_sha256": "0de64d44579c4de69d6dc0e71d3b01ed89c31c3dfbb1a1b784764caa3c0ffd10",
+    "bytes": {"c2": 11694372, "c3": 352653974, "c4": 765471468, "c5": 2181265072},
 }
 
 BENCH_CONFIGS = {

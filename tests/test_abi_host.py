@@ -281,6 +281,7 @@ def test_plan_vectors_per_thread(kw, vpt, threads):
     (dict(nranks=4, tokens=12287, hidden=7168, quant=_capi.QUANT_FP8_TOKEN), 0, (256 * 4 * 8 + 1024) * 4),  # four partials: from 12288
     (dict(nranks=8, tokens=32768, hidden=1024), 4, 39936),                                   # 2 rows x 18 KiB per workgroup
     (dict(nranks=4, tokens=32768, hidden=2048), 6, 26112),
+    (dict(nranks=8, tokens=32768, hidden=2048, dtype=_capi.F64), 0, (1024 * 2 + 1024) * 4),   # doubles: 2 per vector, 1024 threads
     # the per-call override
     (dict(nranks=8, tokens=16, hidden=1024, workgroups_per_cu=1), 1, 162816),
     (dict(nranks=8, tokens=16, hidden=1024, workgroups_per_cu=8), 8, 19456),

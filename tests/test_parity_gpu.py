@@ -437,6 +437,53 @@ def test_static_scale_is_validated(cuda_device):
         assert e.value.status == _capi.EQUANT
 
 
+def test_hip_graph_replays_with_a_workgroup_limit(cuda_device):
+    """A launch limited to two workgroups per CU asks for 79 KiB of dynamic LDS (the kernel's ceiling is raised by the
+    eager warm-up call, before the capture): the captured launch keeps that size and replays with new inputs match the oracle."""
+    dev = cuda_device
+    n, t, h = 4, 96, 7168
+    parts = [torch.empty((t, h), dtype=torch.float16, device=dev) for _ in range(n)]
+    res = torch.empty((t, h), dtype=torch.float16, device=dev)
+    gamma = torch.empty((h,), dtype=torch.float16, device=dev)
+    res_out = torch.empty_like(res)
+    q = torch.empty((t, h), dtype=torch.uint8, device=dev)
+    sc = torch.empty((t, h // 128), dtype=torch.float32, device=dev)
+    prob = _capi.make_problem(_capi.F16, n, t, h, 1e-6, quant=_capi.QUANT_FP8_GROUP, workgroups_per_cu=2)
+    assert _capi.plan(prob).lds_bytes > 64 * 1024
+
+    def launch(stream):
+        _capi.reduce_rms(prob, [p.data_ptr() for p in parts], res.data_ptr(), res_out.data_ptr(), gamma.data_ptr(),
+                         q_out=q.data_ptr(), scale_out=sc.data_ptr(), stream=stream)
+
+    def fill(seed):
+        cp, cr, cg = eager.make_inputs(n, t, h, torch.float16, 1.0, seed=seed)
+        for i in range(n):
+            parts[i].copy_(cp[i])
+        res.copy_(cr)
+        gamma.copy_(cg)
+        return cp, cr, cg
+
+    fill(41)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch(side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        launch(torch.cuda.current_stream().cuda_stream)
+    for seed in (42, 43, 44):
+        cp, cr, cg = fill(seed)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = {"residual_out": res_out.cpu(), "q": q.cpu().view(torch.float8_e4m3fn), "scale": sc.cpu()}
+        for v in (res_out, q, sc):
+            v.zero_()                        # eager work between replays
+        torch.cuda.synchronize()
+        check_against_oracle(got, eager.reduce_rms(cp, cr, cg, 1e-6, "fp8_group"), "fp8_group", gamma=cg, eps=1e-6)
+
+
 @pytest.mark.parametrize("algo", [_capi.ALGO_FUSED, _capi.ALGO_STAGED, _capi.ALGO_STAGED_OWNED])
 def test_hip_graph_replays_match_eager(cuda_device, algo):
     """The launch allocates nothing and synchronizes nothing, so it can be captured (the staged algorithms:

@@ -174,12 +174,9 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
 
     if (geo) {
         geo->wgs_per_cu = wgs_per_cu;
-        geo->lds_bytes = 0;
-        if (p->dtype != TDE_F64) {
-            size_t lds = tde::sumsq_lds_bytes(tpr * rpb, vpt, vec);
-            if (wgs_per_cu > 0) lds = std::max(lds, tde::lds_bytes_for_workgroups_per_cu(wgs_per_cu));
-            geo->lds_bytes = (int)lds;
-        }
+        size_t lds = tde::sumsq_lds_bytes(tpr * rpb, vpt, vec);
+        if (wgs_per_cu > 0) lds = std::max(lds, tde::lds_bytes_for_workgroups_per_cu(wgs_per_cu)); // never with doubles
+        geo->lds_bytes = (int)lds;
         geo->vec_elems = vec;
         geo->nvec = (int)nvec;
         geo->vpt = vpt;

@@ -98,7 +98,7 @@ __global__ void __launch_bounds__(1024) row_kernel_f64(const RowArgs a) {
 
 hipError_t launch_rows_f64(int n, const RowArgs &a, const Geometry &g, hipStream_t s) {
     const dim3 grid((unsigned)g.grid), block((unsigned)g.block_threads);
-    const size_t lds = sumsq_lds_bytes(g.block_threads, 1, 2);
+    const size_t lds = (size_t)g.lds_bytes; // sumsq_lds_bytes(g.block_threads, 1, 2): doubles are never limited per CU
     switch (n) {
     case 2: hipLaunchKernelGGL((row_kernel_f64<2>), grid, block, lds, s, a); break;
     case 4: hipLaunchKernelGGL((row_kernel_f64<4>), grid, block, lds, s, a); break;
