@@ -7,9 +7,11 @@ in HBM.  Inputs and outputs rotate over enough distinct sets (> 4 GiB of inputs,
 outputs) that the 256 MB memory-side cache neither serves a launch's reads nor absorbs its writes.
 The first set is drawn on the CPU from the configuration's seed (the same tensors the parity tests use); the
 CPU-baseline leg runs the oracle on it and compares the kernel's outputs for that set bit for bit.
+Before the W warm-up steps the same step runs untimed for about 20 ms (--settle-ms): a device that has been idle
+runs its first 10-20 ms under load differently from everything after (c3 1 % slower, c5 up to 14 %).
 Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3] [--no-cpu-baseline] [--settle-ms 20]
 """
 import argparse
 import ctypes
@@ -134,6 +136,9 @@ def main():
     ap.add_argument("--sets", type=int, default=0, help="distinct input sets to rotate over (0 = enough for > 1 GiB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--algo", default="auto", choices=["auto", "fused", "staged", "staged_owned"])
+    ap.add_argument("--settle-ms", type=float, default=20.0,
+                    help="before the warm-up steps, run the same step untimed for about this long (0 = not at all; steps shorter "
+                         "than 20 us never): a device that has been idle takes 10-20 ms under load to reach the state it then keeps")
     ap.add_argument("--workgroups-per-cu", type=int, default=0,
                     help="limit on resident workgroups per compute unit: 0 = the library's choice, -1 = none, 1..8 = forced")
     ap.add_argument("--print-source-hash", action="store_true", help="print the kernel-source hash and exit")
@@ -201,8 +206,35 @@ def main():
     call_refs = [ctypes.byref(b) for b in calls]
     hip_stream = ctypes.c_void_p(stream.cuda_stream)
 
+    def settle(fn):
+        """Runs fn(i) back to back, untimed, for about --settle-ms of device time; returns the number of calls.
+        Measured on c3 from a cold process: launches run 57.7-57.9 us for the first 9 ms and 57.0-57.3 us from then
+        on; c5's launches 5 to 50 (2-18 ms) run up to 14 % slow.  A serving process is never in that state."""
+        if args.settle_ms <= 0:
+            return 0
+        for i in range(2):
+            fn(i)
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for i in range(3):
+            fn(i)
+        e1.record(stream)
+        torch.cuda.synchronize(dev)
+        per_call_ms = e0.elapsed_time(e1) / 3
+        if per_call_ms < 0.02:
+            # Launch-bound steps (c2: 5 us) do not load the device, and thousands of them back to back leave the next
+            # 200 anywhere between 5.0 and 6.1 us from one run to the next (0, 1, 3, 8, 20, 60 ms tried): not settled
+            return 0
+        n = int(args.settle_ms / per_call_ms) + 1
+        for i in range(n):
+            fn(i)
+        torch.cuda.synchronize(dev)
+        return n + 5
+
     def timed(fn, steps, warmup):
         """Average duration of `steps` back-to-back calls of fn(i) on the launch stream, by HIP events."""
+        settle(fn)
         for i in range(warmup):
             fn(i)
         torch.cuda.synchronize(dev)
@@ -230,6 +262,7 @@ def main():
     torch.cuda.synchronize(dev)
     del cal_src, cal_dst
 
+    settle_steps = settle(launch)
     for i in range(args.warmup):
         launch(i)
     torch.cuda.synchronize(dev)
@@ -291,6 +324,7 @@ def main():
         "metric": ("achieved HBM GB/s, one rank's 8-partial reduce+residual+RMSNorm+per-token fp8 stage" if args.config == "c3"
                    else "achieved HBM GB/s, one rank's %d-partial reduce+residual+RMSNorm stage, quant=%s" % (N, quant)),
         "value": gbs_job, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "settle_ms": args.settle_ms, "settle_steps": settle_steps,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         # dtype is the arithmetic type (fp32 accumulate, norm and quant); tensors are stored as storage_dtype
         "dtype": "f32", "storage_dtype": dt, "data": "synthetic",
