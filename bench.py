@@ -32,8 +32,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 # They describe the kernels whose sources hash to `sources_sha256`; with any other kernel source the bench line reports
 # traffic as null.
 TRAFFIC = {
-    "sources_sha256": "0de64d44579c4de69d6dc0e71d3b01ed89c31c3dfbb1a1b784764caa3c0ffd10",
-    "bytes": {"c2": 11694372, "c3": 352653974, "c4": 765471468, "c5": 2181265072},
+    "sources_sha256": "2a8023f541678c8960c597ab3b21800ab99b1e515f6fd7be746be100c695cdbb",
+    "bytes": {"c2": 11695287, "c3": 352653932, "c4": 765468035, "c5": 2181276242},
 }
 
 BENCH_CONFIGS = {

@@ -62,8 +62,9 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 constexpr int kMaxBlock = 1024;
 constexpr int64_t kLoadsInFlightPerCu = 128 * 1024; // target for the limit on resident workgroups (see validate)
-// launches with fewer workgroups are not limited (8 partials; twice as many with 4, whose launches are half as long)
-constexpr int64_t kLimitWorkgroupsFromGrid = 6144;
+// launches with fewer workgroups per compute unit are not limited (8 partials; twice as many with 4, whose launches are
+// half as long): 6144 and 12288 workgroups on the 256 CUs of an unpartitioned MI355X
+constexpr int64_t kLimitFromWorkgroupsPerCu = 24;
 constexpr int kDefaultComputeUnits = 256; // MI355X; used when no device can be asked (planning on a host without one)
 
 // Compute units of the current device, asked once per device.
@@ -162,7 +163,7 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     // few generations of workgroups) gain nothing and can lose 1-3 %, and with 2 partials no limit helps.
     int wgs_per_cu = 0;
     const bool staged = p->algo == TDE_ALGO_STAGED || p->algo == TDE_ALGO_STAGED_OWNED; // its row kernel reads 2 streams
-    if (p->dtype != TDE_F64 && !staged && p->nranks >= 4 && grid >= kLimitWorkgroupsFromGrid * (p->nranks >= 8 ? 1 : 2)) {
+    if (p->dtype != TDE_F64 && !staged && p->nranks >= 4 && grid >= kLimitFromWorkgroupsPerCu * cus * (p->nranks >= 8 ? 1 : 2)) {
         const int64_t per_wg = (int64_t)rpb * (p->nranks + 1) * nvec * 16; // bytes of loads one workgroup keeps in flight
         const int waves = tpr * rpb / 64;
         // per-group scales are the heaviest arithmetic per row and four partials the shortest loads to cover it
