@@ -437,6 +437,36 @@ def test_static_scale_is_validated(cuda_device):
         assert e.value.status == _capi.EQUANT
 
 
+def test_first_large_lds_launch_inside_a_capture(cuda_device):
+    """The first launch of a kernel with more than 64 KiB of dynamic LDS raises that kernel's ceiling (a function
+    attribute, not a stream operation).  No other test launches this instantiation (fp32, 2 partials, int8) with such a
+    size, so here that happens while the stream is being captured; the graph must still be valid and right."""
+    dev = cuda_device
+    n, t, h = 2, 64, 2048
+    cp, cr, cg = eager.make_inputs(n, t, h, torch.float32, 1.0, seed=5)
+    parts = [p.to(dev) for p in cp]
+    res, gamma = cr.to(dev), cg.to(dev)
+    res_out = torch.empty_like(res)
+    q = torch.empty((t, h), dtype=torch.uint8, device=dev)
+    sc = torch.empty((t,), dtype=torch.float32, device=dev)
+    prob = _capi.make_problem(_capi.F32, n, t, h, 1e-6, quant=_capi.QUANT_INT8_TOKEN, workgroups_per_cu=1)
+    assert _capi.plan(prob).lds_bytes > 64 * 1024
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        _capi.reduce_rms(prob, [p.data_ptr() for p in parts], res.data_ptr(), res_out.data_ptr(), gamma.data_ptr(),
+                         q_out=q.data_ptr(), scale_out=sc.data_ptr(), stream=torch.cuda.current_stream().cuda_stream)
+    want = eager.reduce_rms(cp, cr, cg, 1e-6, "int8_token")
+    for _ in range(2):
+        for v in (res_out, q, sc):
+            v.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = {"residual_out": res_out.cpu(), "q": q.cpu().view(torch.int8), "scale": sc.cpu()}
+        check_against_oracle(got, want, "int8_token", gamma=cg, eps=1e-6)
+
+
 def test_hip_graph_replays_with_a_workgroup_limit(cuda_device):
     """A launch limited to two workgroups per CU asks for 79 KiB of dynamic LDS (the kernel's ceiling is raised by the
     eager warm-up call, before the capture): the captured launch keeps that size and replays with new inputs match the oracle."""
