@@ -614,6 +614,31 @@ def test_randomized_shapes_and_modes(cuda_device):
     assert done == 64
 
 
+def test_randomized_launch_geometries(cuda_device):
+    """The same kind of sweep with the launch forced at random as well: vectors per thread, rows per workgroup, the
+    limit on workgroups per CU (with and without more than 64 KiB of LDS), the algorithm and the extra normed output."""
+    rng = torch.Generator().manual_seed(77)
+
+    def pick(seq):
+        return seq[int(torch.randint(0, len(seq), (1,), generator=rng))]
+
+    for k in range(48):
+        dtype = pick([torch.bfloat16, torch.float16, torch.float32])
+        n = pick([2, 4, 8])
+        tokens = int(torch.randint(1, 50, (1,), generator=rng))
+        vec = 4 if dtype == torch.float32 else 8
+        quant = pick(["none", "fp8_token", "fp8_group", "int8_token"])
+        hidden = int(torch.randint(1, 1025, (1,), generator=rng)) * vec
+        if quant == "fp8_group":
+            hidden = max(128, hidden // 128 * 128)
+        kw = dict(vecs_per_thread=pick([0, 1, 2, 4]), rows_per_block=pick([0, 0, 1, 2, 4]),
+                  workgroups_per_cu=pick([0, -1, 1, 2, 3, 5, 8]), algo=pick([_capi.ALGO_AUTO, _capi.ALGO_AUTO, _capi.ALGO_STAGED]),
+                  write_norm=pick([True, False]))
+        p, r, g = eager.make_inputs(n, tokens, hidden, dtype, 1.0, seed=2000 + k)
+        print("geometry fuzz", k, dtype, n, tokens, hidden, quant, kw, flush=True)
+        _case("geofuzz%d" % k, p, r, g, 1e-6, quant, **kw)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("scale", [1e-30, 3e-39, 1e-6, 1e4])
 def test_extreme_magnitudes(cuda_device, dtype, scale):
