@@ -32,8 +32,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 # They describe the kernels whose sources hash to `sources_sha256`; with any other kernel source the bench line reports
 # traffic as null.
 TRAFFIC = {
-    "sources_sha256": "2a8023f541678c8960c597ab3b21800ab99b1e515f6fd7be746be100c695cdbb",
-    "bytes": {"c2": 11695287, "c3": 352653932, "c4": 765468035, "c5": 2181276242},
+    "sources_sha256": "83fc4b01bcba134fe66bbedb518b7eb987f60f614962844edf2984a0b67b1734",
+    "bytes": {"c2": 11694347, "c3": 352654238, "c4": 765471037, "c5": 2181253551},
 }
 
 BENCH_CONFIGS = {

@@ -276,9 +276,9 @@ def test_plan_vectors_per_thread(kw, vpt, threads):
     (dict(nranks=8, tokens=6144, hidden=8192), 2, 80896),                                    # 144 KiB per workgroup
     (dict(nranks=4, tokens=32768, hidden=8192), 2, 80896),                                   # 80 KiB per workgroup
     (dict(nranks=4, tokens=32768, hidden=5120, dtype=_capi.F16, quant=_capi.QUANT_INT8_TOKEN), 3, 53504),  # 3 wavefronts each
-    (dict(nranks=4, tokens=12288, hidden=7168, quant=_capi.QUANT_FP8_GROUP), 3, 53504),     # twelve wavefronts for group scales
-    (dict(nranks=4, tokens=12288, hidden=7168, quant=_capi.QUANT_FP8_TOKEN), 2, 80896),
-    (dict(nranks=4, tokens=12287, hidden=7168, quant=_capi.QUANT_FP8_TOKEN), 0, (256 * 4 * 8 + 1024) * 4),  # four partials: from 12288
+    (dict(nranks=4, tokens=8192, hidden=7168, quant=_capi.QUANT_FP8_GROUP), 3, 53504),      # twelve wavefronts for group scales
+    (dict(nranks=4, tokens=8192, hidden=7168, quant=_capi.QUANT_FP8_TOKEN), 2, 80896),
+    (dict(nranks=4, tokens=8191, hidden=7168, quant=_capi.QUANT_FP8_TOKEN), 0, (256 * 4 * 8 + 1024) * 4),   # four partials: from 8192
     (dict(nranks=8, tokens=32768, hidden=1024), 4, 39936),                                   # 2 rows x 18 KiB per workgroup
     (dict(nranks=4, tokens=32768, hidden=2048), 6, 26112),
     (dict(nranks=8, tokens=32768, hidden=2048, dtype=_capi.F64), 0, (1024 * 2 + 1024) * 4),   # doubles: 2 per vector, 1024 threads

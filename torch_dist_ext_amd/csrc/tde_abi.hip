@@ -62,9 +62,9 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 constexpr int kMaxBlock = 1024;
 constexpr int64_t kLoadsInFlightPerCu = 128 * 1024; // target for the limit on resident workgroups (see validate)
-// launches with fewer workgroups per compute unit are not limited (8 partials; twice as many with 4, whose launches are
-// half as long): 6144 and 12288 workgroups on the 256 CUs of an unpartitioned MI355X
-constexpr int64_t kLimitFromWorkgroupsPerCu = 24;
+// launches with fewer workgroups per compute unit are not limited: 24 with 8 partials, 32 with 4 (whose launches are
+// shorter), i.e. 6144 and 8192 workgroups on the 256 CUs of an unpartitioned MI355X
+constexpr int64_t kLimitFromWorkgroupsPerCu8 = 24, kLimitFromWorkgroupsPerCu4 = 32;
 constexpr int kDefaultComputeUnits = 256; // MI355X; used when no device can be asked (planning on a host without one)
 
 // Compute units of the current device, asked once per device.
@@ -160,10 +160,12 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     // of loads in flight per CU: more costs 1-8 % from 8192 rows up with 4 or 8 partials (32768 x 8192: 7.5 % with
     // 4 partials, 4.5 % with 8; 16384 rows: 1-3 %; 8192 rows with 8 partials: 1 %), fewer than two workgroups or
     // eight wavefronts per CU leave the arithmetic of one row uncovered by the loads of another.  Short launches (a
-    // few generations of workgroups) gain nothing and can lose 1-3 %, and with 2 partials no limit helps.
+    // few generations of workgroups) gain nothing and can lose 1-3 %, and with 2 partials no limit helps.  At the
+    // threshold itself the gain is small: 4 x [8192, 7168] with per-group scales 0.4 % on a device that has been under
+    // load for 20 ms (0.9 % slower in the first milliseconds after idling).
     int wgs_per_cu = 0;
     const bool staged = p->algo == TDE_ALGO_STAGED || p->algo == TDE_ALGO_STAGED_OWNED; // its row kernel reads 2 streams
-    if (p->dtype != TDE_F64 && !staged && p->nranks >= 4 && grid >= kLimitFromWorkgroupsPerCu * cus * (p->nranks >= 8 ? 1 : 2)) {
+    if (p->dtype != TDE_F64 && !staged && p->nranks >= 4 && grid >= (p->nranks >= 8 ? kLimitFromWorkgroupsPerCu8 : kLimitFromWorkgroupsPerCu4) * cus) {
         const int64_t per_wg = (int64_t)rpb * (p->nranks + 1) * nvec * 16; // bytes of loads one workgroup keeps in flight
         const int waves = tpr * rpb / 64;
         // per-group scales are the heaviest arithmetic per row and four partials the shortest loads to cover it
