@@ -29,6 +29,7 @@ namespace tde {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -82,6 +83,8 @@ struct ElemBF16 {
         }
         return raw;
     }
+    // fp32 bit pattern of a non-negative element given by its own bits
+    static __device__ __forceinline__ uint32_t magnitude_to_f32_bits(uint32_t m) { return m << 16; }
 };
 
 struct ElemF16 {
@@ -105,6 +108,9 @@ struct ElemF16 {
         }
         return raw;
     }
+    static __device__ __forceinline__ uint32_t magnitude_to_f32_bits(uint32_t m) {
+        return __builtin_bit_cast(uint32_t, (float)__builtin_bit_cast(_Float16, (uint16_t)m)); // NaN stays NaN
+    }
 };
 
 struct ElemF32 {
@@ -123,28 +129,57 @@ struct ElemF32 {
         for (int i = 0; i < 4; ++i) raw[i] = __builtin_bit_cast(uint32_t, f[i]);
         return raw;
     }
+    static __device__ __forceinline__ uint32_t magnitude_to_f32_bits(uint32_t m) { return m; }
 };
+
+// Largest magnitude of a row's elements, taken on the bit patterns: for non-negative floats of one format the
+// unsigned order of the bits is the order of the values with every NaN above infinity, so an unsigned maximum of
+// |x| propagates NaN as torch's amax does (a float maximum would drop it) and costs no more.  The 2-byte types keep
+// two running 16-bit maxima in one register (one packed instruction per two elements).
+//   amax_fold: folds a 16-byte vector into the running maximum (start from 0)
+//   amax_f32_bits: the fp32 bit pattern of the largest magnitude folded in (a NaN pattern if any element was NaN)
+__device__ __forceinline__ uint32_t max_u32(uint32_t a, uint32_t b) { return a > b ? a : b; }
+
+template <class E>
+__device__ __forceinline__ uint32_t amax_fold(uint32_t acc, u32x4 raw) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t w = raw[i]; // copy first: bit_cast applied straight to a vector element reads lane 0
+        if constexpr (E::BYTES == 2) {
+            const u16x2 a = __builtin_bit_cast(u16x2, acc), b = __builtin_bit_cast(u16x2, w & 0x7fff7fffu);
+            acc = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
+        } else {
+            acc = max_u32(acc, w & 0x7fffffffu);
+        }
+    }
+    return acc;
+}
+
+template <class E>
+__device__ __forceinline__ uint32_t amax_f32_bits(uint32_t acc) {
+    if constexpr (E::BYTES == 2) acc = max_u32(acc >> 16, acc & 0xffffu);
+    return E::magnitude_to_f32_bits(acc);
+}
 
 // ---------------------------------------------------------------------------------------------
 // 64-lane wavefront reductions: four DPP steps inside each 16-lane row, then the four row
 // results are combined through v_readlane.  Every lane ends with the same value.
 // ---------------------------------------------------------------------------------------------
 template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_move_u32(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+}
+template <int CTRL>
 __device__ __forceinline__ float dpp_move(float v) {
-    return __builtin_bit_cast(
-        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+    return __builtin_bit_cast(float, dpp_move_u32<CTRL>(__builtin_bit_cast(uint32_t, v)));
 }
 
-struct OpMax {
-    static __device__ __forceinline__ float f(float a, float b) { return fmaxf(a, b); }
-};
-
-template <class Op>
-__device__ __forceinline__ float row16_reduce(float v) {
-    v = Op::f(v, dpp_move<0xB1>(v));  // quad_perm [1,0,3,2]
-    v = Op::f(v, dpp_move<0x4E>(v));  // quad_perm [2,3,0,1]
-    v = Op::f(v, dpp_move<0x141>(v)); // row_half_mirror
-    v = Op::f(v, dpp_move<0x140>(v)); // row_mirror
+// Unsigned maximum over each 16-lane row (the maxima here are bit patterns of magnitudes, see amax_fold).
+__device__ __forceinline__ uint32_t row16_max(uint32_t v) {
+    v = max_u32(v, dpp_move_u32<0xB1>(v));  // quad_perm [1,0,3,2]
+    v = max_u32(v, dpp_move_u32<0x4E>(v));  // quad_perm [2,3,0,1]
+    v = max_u32(v, dpp_move_u32<0x141>(v)); // row_half_mirror
+    v = max_u32(v, dpp_move_u32<0x140>(v)); // row_mirror
     return v;
 }
 
@@ -152,25 +187,23 @@ __device__ __forceinline__ float read_lane(float v, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
 
-template <class Op>
-__device__ __forceinline__ float wave_reduce(float v) {
-    v = row16_reduce<Op>(v);
-    const float a = read_lane(v, 0), b = read_lane(v, 16), c = read_lane(v, 32), d = read_lane(v, 48);
-    return Op::f(Op::f(a, b), Op::f(c, d));
+__device__ __forceinline__ uint32_t wave_max(uint32_t v) {
+    v = row16_max(v);
+    const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16),
+                   c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    return max_u32(max_u32(a, b), max_u32(c, d));
 }
 
-// Reduce over the `waves_per_row` wavefronts that share a row.  `slots` is an LDS buffer indexed by wavefront
-// number inside the block, used once per kernel (one barrier).  Identity is 0 (maxima of absolute values).
-template <class Op>
-__device__ __forceinline__ float row_reduce(float v, float *slots, int wave, int lane, int first_wave,
-                                            int waves_per_row) {
-    v = wave_reduce<Op>(v);
+// Maximum over the `waves_per_row` wavefronts that share a row.  `slots` is an LDS buffer indexed by wavefront
+// number inside the block, used once per kernel (one barrier).  Identity is 0 (bit patterns of magnitudes).
+__device__ __forceinline__ uint32_t row_max(uint32_t v, uint32_t *slots, int wave, int lane, int first_wave, int waves_per_row) {
+    v = wave_max(v);
     if (waves_per_row == 1) return v;
     if (lane == 0) slots[wave] = v;
     __syncthreads();
     const int k = lane & 15;
-    const float t = (k < waves_per_row) ? slots[first_wave + k] : 0.0f;
-    return row16_reduce<Op>(t);
+    const uint32_t t = (k < waves_per_row) ? slots[first_wave + k] : 0u;
+    return row16_max(t);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -447,10 +480,18 @@ __device__ __forceinline__ void pack_int8(const float (&q)[VEC], uint32_t (&out)
 // in one fma; adding residual*rcp back in a second fma rounds to the correctly rounded quotient
 // (Markstein's division theorem) as long as nothing underflows.  Callers take this path only when
 // d is far from the subnormal and overflow ranges and use a plain division otherwise.
+// The residual is taken as q0*d - y and subtracted, not as y - q0*d and added: the same value for every non-zero y,
+// and for y = -0 the result is then -0 like the quotient's (the other form ends in (+0) + (-0) = +0).
 __device__ __forceinline__ float div_shared(float y, float d, float rcp) {
     const float q0 = y * rcp;
-    const float e = __builtin_fmaf(-q0, d, y);
-    return __builtin_fmaf(e, rcp, q0);
+    const float e = __builtin_fmaf(q0, d, -y);
+    return __builtin_fmaf(-e, rcp, q0);
+}
+
+// min(max(q, -limit), limit) that keeps NaN, as torch.clamp does (the float minimum and maximum drop it).
+__device__ __forceinline__ float clamp_keep_nan(float q, float limit) {
+    const float c = fminf(fmaxf(q, -limit), limit);
+    return (q != q) ? q : c;
 }
 
 // Which row group a workgroup takes.  Workgroups are handed to the 8 XCDs round-robin, so in launch order
@@ -500,7 +541,7 @@ __global__ void __launch_bounds__(1024 / VPT)
     extern __shared__ __attribute__((aligned(16))) float lds_dyn[];
     float *const lds_img = lds_dyn;
     float *const lds_bs = lds_dyn + blockDim.x * (VPT * VEC);
-    __shared__ float lds_max[kMaxWavesPerBlock];
+    __shared__ uint32_t lds_max[kMaxWavesPerBlock];
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -656,7 +697,7 @@ __global__ void __launch_bounds__(1024 / VPT)
 
         // ---- normalize ------------------------------------------------------------------------------
         u32x4 yraw[VPT];
-        float amax[VPT];
+        uint32_t amax[VPT]; // running maxima of the magnitudes' bit patterns (amax_fold), per vector
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
             float x[VEC], g[VEC], y[VEC];
@@ -672,13 +713,7 @@ __global__ void __launch_bounds__(1024 / VPT)
                 const rsrc_t norm_out = row_rsrc(a.norm_out, row_byte, bytes);
                 rsrc_store16(norm_out, TDE_OFF(j), yraw[j]);
             }
-            if constexpr (Q != TDE_QUANT_NONE && Q != TDE_QUANT_FP8_STATIC) {
-                E::unpack(yraw[j], y);
-                float m = 0.0f;
-#pragma unroll
-                for (int i = 0; i < VEC; ++i) m = fmaxf(m, __builtin_fabsf(y[i]));
-                amax[j] = m;
-            }
+            if constexpr (Q != TDE_QUANT_NONE && Q != TDE_QUANT_FP8_STATIC) amax[j] = amax_fold<E>(0u, yraw[j]);
         }
 
         if constexpr (Q == TDE_QUANT_NONE) {
@@ -696,9 +731,9 @@ __global__ void __launch_bounds__(1024 / VPT)
                 const rsrc_t sc_out = row_rsrc(a.scale_out, row * groups_per_row * 4, row_ok ? (uint32_t)groups_per_row * 4u : 0u);
 #pragma unroll
                 for (int j = 0; j < VPT; ++j) {
-                    float m = row16_reduce<OpMax>(amax[j]);
-                    if constexpr (LANES_PER_GROUP == 32) m = fmaxf(m, __shfl_xor(m, 16, kWave));
-                    scale[j] = m / QMAX;
+                    uint32_t m = row16_max(amax_f32_bits<E>(amax[j]));
+                    if constexpr (LANES_PER_GROUP == 32) m = max_u32(m, (uint32_t)__shfl_xor((int)m, 16, kWave));
+                    scale[j] = __builtin_bit_cast(float, m) / QMAX;
                     if ((TDE_LANE & (LANES_PER_GROUP - 1)) == 0)
                         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, scale[j]), sc_out,
                                                               (int)((TDE_OFF(j) / 16u / LANES_PER_GROUP) * 4u), 0, kAuxDefault);
@@ -707,11 +742,14 @@ __global__ void __launch_bounds__(1024 / VPT)
 #pragma unroll
                 for (int j = 0; j < VPT; ++j) scale[j] = a.static_scale;
             } else {
-                float m = amax[0];
+                uint32_t m = amax[0];
 #pragma unroll
-                for (int j = 1; j < VPT; ++j) m = fmaxf(m, amax[j]);
-                m = row_reduce<OpMax>(m, lds_max, wave, TDE_LANE, first_wave, waves_per_row);
-                const float sc = m / QMAX;
+                for (int j = 1; j < VPT; ++j) {
+                    if constexpr (E::BYTES == 2) m = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, m), __builtin_bit_cast(u16x2, amax[j])));
+                    else m = max_u32(m, amax[j]);
+                }
+                m = row_max(amax_f32_bits<E>(m), lds_max, wave, TDE_LANE, first_wave, waves_per_row);
+                const float sc = __builtin_bit_cast(float, m) / QMAX;
 #pragma unroll
                 for (int j = 0; j < VPT; ++j) scale[j] = sc;
                 if (row_ok && TDE_T == 0) ((TDE_GLOBAL float *)a.scale_out)[row] = sc;
@@ -720,13 +758,11 @@ __global__ void __launch_bounds__(1024 / VPT)
 #pragma unroll
             for (int j = 0; j < VPT; ++j) rsrc_store16(res_out, TDE_OFF(j), xraw[j]);
             // One wavefront-uniform decision for all of the thread's vectors, so the common path carries no per-lane
-            // branch: the fast quotient needs every divisor far from the subnormal and overflow ranges.
+            // branch: the fast quotient needs every divisor far from the subnormal and overflow ranges.  A dynamic scale
+            // that is NaN or infinite (a NaN or an infinity among the normed values) also takes the plain division.
             bool unsafe = false;
 #pragma unroll
-            for (int j = 0; j < VPT; ++j) {
-                const float div = (scale[j] > 0.0f) ? scale[j] : 1.0f;
-                unsafe = unsafe || !(div > 0x1p-60f && div < 0x1p60f);
-            }
+            for (int j = 0; j < VPT; ++j) unsafe = unsafe || !(scale[j] == 0.0f || (scale[j] > 0x1p-60f && scale[j] < 0x1p60f));
             const bool fast = __builtin_amdgcn_ballot_w64(unsafe) == 0;
             auto quantize = [&](auto use_fast) {
 #pragma unroll
@@ -740,15 +776,22 @@ __global__ void __launch_bounds__(1024 / VPT)
                         // there: the product y * rcp then stays finite and the correction never sees inf - inf.
                         const float ymax = (div < 0x1p60f) ? 2.0f * QMAX * div : 3.0e38f;
 #pragma unroll
-                        for (int i = 0; i < VEC; ++i) y[i] = fminf(fmaxf(y[i], -ymax), ymax);
+                        for (int i = 0; i < VEC; ++i) y[i] = clamp_keep_nan(y[i], ymax);
                     }
                     if constexpr (decltype(use_fast)::value) {
                         const float rcp = 1.0f / div;
+                        if constexpr (Q == TDE_QUANT_FP8_STATIC) {
 #pragma unroll
-                        for (int i = 0; i < VEC; ++i) q[i] = fminf(fmaxf(div_shared(y[i], div, rcp), -QMAX), QMAX);
+                            for (int i = 0; i < VEC; ++i) q[i] = clamp_keep_nan(div_shared(y[i], div, rcp), QMAX);
+                        } else {
+                            // |y| <= QMAX * scale up to two roundings: the quotient is within 1e-4 of +-QMAX at most,
+                            // which the conversions below round to the largest code; nothing to clamp
+#pragma unroll
+                            for (int i = 0; i < VEC; ++i) q[i] = div_shared(y[i], div, rcp);
+                        }
                     } else {
 #pragma unroll
-                        for (int i = 0; i < VEC; ++i) q[i] = fminf(fmaxf(y[i] / div, -QMAX), QMAX);
+                        for (int i = 0; i < VEC; ++i) q[i] = clamp_keep_nan(y[i] / div, QMAX);
                     }
                     uint32_t codes[VEC / 4];
                     if constexpr (Q == TDE_QUANT_INT8_TOKEN)
