@@ -42,7 +42,7 @@ typedef enum tde_status {
     TDE_EALIGN = 6,     /* a buffer is not 16-byte aligned (vec_t alignment, impl.h:208) */
     TDE_EQUANT = 7,     /* unknown quant mode, group mode with hidden % 128 != 0, a static scale that is not > 0,
                            or any quant mode with TDE_F64 */
-    TDE_EALGO = 8,      /* unknown algorithm, staged algorithm without a stage buffer or with TDE_F64 */
+    TDE_EALGO = 8,      /* unknown algorithm, or staged algorithm without a stage buffer */
     TDE_EHIP = 9,       /* HIP runtime error; see tde_last_hip_error() */
     TDE_ERANK = 10,     /* rank outside [0,nranks) */
     TDE_ENOMEM = 11,    /* device allocation failed */
@@ -56,7 +56,7 @@ typedef enum tde_dtype {
     TDE_F32 = 2,  /* float,                               src/ops/all_reduce_fusion.cpp:29-33 */
     TDE_F64 = 3   /* double, admitted by the same macro;  src/ops/all_reduce_fusion.cpp:29-33.  Summed and normed
                      in double as the eager composition does for double tensors (mean of squares in fp32,
-                     test_all_reduce_fusion.py:25); TDE_QUANT_NONE and the fused algorithm only */
+                     test_all_reduce_fusion.py:25); TDE_QUANT_NONE only, every algorithm */
 } tde_dtype;
 
 typedef enum tde_quant {
@@ -131,7 +131,9 @@ typedef struct tde_plan_out {
     int32_t grid_blocks;     /* workgroups launched for the row kernel */
     int32_t xcd_chunk;       /* row groups each XCD takes in a row: workgroup b of every 8*xcd_chunk takes row group
                                 (b % 8) * xcd_chunk + b / 8 of that span (1 = launch order) */
-    int32_t workgroups_per_cu; /* limit on resident workgroups per compute unit the launch enforces (0 = none) */
+    int32_t workgroups_per_cu; /* limit on resident workgroups per compute unit the launch enforces through its LDS
+                                  (0 = none); below a requested tune_workgroups_per_cu where the geometry's own LDS
+                                  already admits fewer */
     int32_t lds_bytes;         /* dynamic LDS per workgroup of the row kernel's launch, padding included */
     int64_t algorithmic_bytes; /* (N+1)*T*H*e + H*e + T*H*e + OUT, OUT as documented for the quant mode */
     int64_t scale_elems;       /* number of fp32 scales written */

@@ -37,6 +37,30 @@ def bits_equal(a: torch.Tensor, b: torch.Tensor) -> bool:
     return va.shape == vb.shape and bool(torch.equal(va, vb))
 
 
+def equal_where_not_nan(got: torch.Tensor, want: torch.Tensor, nan_codes=False, ignore=None) -> bool:
+    """Bit equality of two tensors of one dtype, except that a NaN matches any NaN: which NaN comes out of inf - inf
+    or of a conversion (sign, payload) is the processor's choice (x86 makes 0xFFC00000, gfx950 0x7FC00000) and not part
+    of the contract.  nan_codes: the tensors hold e4m3 codes (0x7F and 0xFF are NaN).  ignore: boolean mask of
+    elements left out of the comparison."""
+    if got.shape != want.shape or got.dtype != want.dtype:
+        return False
+    if nan_codes:
+        g, w = got.view(torch.uint8), want.view(torch.uint8)
+        gn, wn = (g & 0x7F) == 0x7F, (w & 0x7F) == 0x7F
+        same = g == w
+    else:
+        gn, wn = torch.isnan(got), torch.isnan(want)
+        if got.element_size() == 8:
+            same = got.view(torch.int64) == want.view(torch.int64)
+        else:
+            view = {1: torch.uint8, 2: torch.int16, 4: torch.int32}[got.element_size()]
+            same = got.view(view) == want.view(view)
+    ok = (gn & wn) | (same & ~gn & ~wn)
+    if ignore is not None:
+        ok = ok | ignore
+    return bool(ok.all())
+
+
 def run_hip(parts, residual, gamma, eps, quant="none", algo=_capi.ALGO_AUTO, write_norm=None, use_table=False,
             rank=0, device="cuda:0", static_scale=0.0, stage_init=None, calls=None, vecs_per_thread=0, rows_per_block=0,
             workgroups_per_cu=0):
@@ -148,7 +172,41 @@ def quant_from_own_norm(norm_got, quant):
     return eager.quant_int8(norm_got)
 
 
-def check_against_oracle(got, want, quant, gamma=None, eps=None, strict=True):
+_SUM_ORDER_PINNED = None
+
+
+def torch_sum_order_is_pinned() -> bool:
+    """Does this host's torch sum a contiguous fp32 row in the order the kernel follows?  Probed once per process
+    on the CPU: the C restatement of that order (oracle/tde_oracle.c: tdo_torch_row_sum) against torch.sum on fixed
+    seeded rows of several lengths (left-over vectors and scalars included).  The order belongs to torch's CPU
+    reduction kernel, which the reference does not pin; when a host's torch sums differently the bit-for-bit
+    comparison of norm_out, scales and codes would report a host change as a kernel regression, so
+    check_against_oracle then falls back to the stated bounds (and says so)."""
+    global _SUM_ORDER_PINNED
+    if _SUM_ORDER_PINNED is None:
+        import warnings
+        try:
+            from oracle import cport
+            g = torch.Generator().manual_seed(20240607)
+            ok = True
+            for n in (8192, 7168, 5120, 4096, 1000, 508, 124, 37):
+                x = torch.randn((5, n), generator=g, dtype=torch.float32).pow(2)
+                mine = torch.from_numpy(cport.torch_row_sums(x.numpy()))
+                ok = ok and bool(torch.equal(mine.view(torch.int32), x.sum(dim=-1).view(torch.int32)))
+            _SUM_ORDER_PINNED = ok
+        except Exception as e:   # no C oracle built: nothing to probe with, keep the strict comparison
+            warnings.warn("sum-order probe unavailable (%s); comparing bit for bit" % e)
+            _SUM_ORDER_PINNED = True
+        if not _SUM_ORDER_PINNED:
+            warnings.warn("this host's torch does not sum rows in the pinned order: norm_out, scales and codes are "
+                          "compared within the stated bounds (1 ulp, 1 quant step, 1e-6), not bit for bit")
+        print("check_against_oracle: %s comparison (torch CPU sum order %s)" % (
+            "bit-for-bit" if _SUM_ORDER_PINNED else "bounded", "as pinned" if _SUM_ORDER_PINNED else "DIFFERS from the pin"),
+            flush=True)
+    return _SUM_ORDER_PINNED
+
+
+def check_against_oracle(got, want, quant, gamma=None, eps=None, strict=None):
     """Every output bit for bit against the oracle's.
 
     residual_out: fp32 rank-order sum, one rounding, residual add, one rounding (bit-exact by contract).
@@ -160,8 +218,11 @@ def check_against_oracle(got, want, quant, gamma=None, eps=None, strict=True):
 
     strict=False relaxes norm_out/scales/codes to those stated bounds plus the allowance for a reciprocal RMS that
     differs in its last bit (for a host whose torch sums in another order); the stage-exact checks stay.
-    Returns mismatch statistics (all zero when strict)."""
-    stats = {}
+    strict=None (the default) chooses: bit for bit where this host's torch sums in the pinned order
+    (torch_sum_order_is_pinned), the bounds otherwise.  Returns mismatch statistics (all zero when strict)."""
+    if strict is None:
+        strict = torch_sum_order_is_pinned()
+    stats = {"strict": bool(strict)}
     assert bits_equal(got["residual_out"], want["residual_out"]), "residual_out is not bit-exact"
     flipped = 0
     if "norm_out" in got:

@@ -459,3 +459,16 @@ def test_doubles_are_summed_as_doubles():
     assert y.dtype == torch.float64
     assert abs(y[0, 0].item() - 6.0 * rs) < 1e-6 and abs(y[0, 1].item() - 2.0 * rs) < 1e-6
     assert y[0, 0].item() == 2.0 * (3.0 * float(torch.rsqrt(torch.tensor(12.5, dtype=torch.float32))))
+
+
+def test_strictness_of_the_gpu_comparison_follows_the_sum_order_probe(monkeypatch):
+    """helpers.check_against_oracle compares bit for bit only where this host's torch sums rows in the pinned order
+    (probed once per process); otherwise it falls back to the stated bounds instead of reporting a host change as a
+    kernel regression.  Here the order is the pinned one, and a forced negative probe selects the bounded mode."""
+    import helpers
+    assert helpers.torch_sum_order_is_pinned() is True
+    p, r, g = eager.make_inputs(4, 5, 256, torch.bfloat16, 1.0, seed=3)
+    want = eager.reduce_rms(p, r, g, 1e-6, "fp8_token")
+    assert helpers.check_against_oracle(dict(want), want, "fp8_token", gamma=g, eps=1e-6)["strict"] is True
+    monkeypatch.setattr(helpers, "_SUM_ORDER_PINNED", False)
+    assert helpers.check_against_oracle(dict(want), want, "fp8_token", gamma=g, eps=1e-6)["strict"] is False

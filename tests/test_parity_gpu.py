@@ -10,12 +10,12 @@ import torch
 from oracle import eager
 from torch_dist_ext_amd import _capi
 
-from helpers import bits_equal, check_against_oracle, run_hip, ulp_distance
+from helpers import bits_equal, check_against_oracle, equal_where_not_nan, run_hip, ulp_distance
 
 pytestmark = pytest.mark.gpu
 
 
-def _case(name, parts, residual, gamma, eps, quant, strict=True, **kw):
+def _case(name, parts, residual, gamma, eps, quant, strict=None, **kw):
     print("case", name, tuple(parts.shape), residual.dtype, quant, kw, flush=True)
     want = eager.reduce_rms(parts, residual, gamma, eps, quant)
     got = run_hip(parts, residual, gamma, eps, quant, **kw)
@@ -65,6 +65,8 @@ def test_staged_equals_fused(cuda_device, quant):
     b = run_hip(p, r, g, 1e-6, quant, algo=_capi.ALGO_STAGED)
     for k in a:
         assert bits_equal(a[k], b[k]), k
+    # and the staged outputs against the oracle themselves, not only against the fused kernel
+    check_against_oracle(b, eager.reduce_rms(p, r, g, 1e-6, quant), quant, gamma=g, eps=1e-6)
 
 
 def _rank_order_sum(parts):
@@ -97,6 +99,7 @@ def test_staged_owned_rows(cuda_device, n, rank, tokens, hidden, dtype, quant):
     assert bits_equal(b.pop("stage"), sums)
     for k in a:
         assert bits_equal(a[k], b[k]), k
+    check_against_oracle(b, eager.reduce_rms(p, r, g, 1e-6, quant), quant, gamma=g, eps=1e-6)
     # a wrong share is visible: with nothing pre-filled, rows of other ranks stay NaN
     if tokens > 1:
         c = run_hip(p, r, g, 1e-6, quant, algo=_capi.ALGO_STAGED_OWNED, rank=rank,
@@ -124,10 +127,13 @@ def test_two_shot_emulated_by_phase_calls(cuda_device, n, tokens, hidden, dtype,
     assert bits_equal(b.pop("stage"), _rank_order_sum(p))
     for k in a:
         assert bits_equal(a[k], b[k]), k
+    want = eager.reduce_rms(p, r, g, 1e-6, quant)
+    check_against_oracle(b, want, quant, gamma=g, eps=1e-6)
     # and the all-rows staged algorithm split the same way
     c = run_hip(p, r, g, 1e-6, quant, algo=_capi.ALGO_STAGED, calls=[(("reduce",), 0), (("norm",), 0)])
     for k in a:
         assert bits_equal(a[k], c[k]), k
+    check_against_oracle(c, want, quant, gamma=g, eps=1e-6)
 
 
 def test_phase_calls_need_a_staged_algorithm(cuda_device):
@@ -639,6 +645,88 @@ def test_randomized_launch_geometries(cuda_device):
         _case("geofuzz%d" % k, p, r, g, 1e-6, quant, **kw)
 
 
+def _check_nonfinite(got, want, quant, static_scale=None):
+    """Every output against the oracle's with NaN matching NaN (helpers.equal_where_not_nan); int8 codes are left
+    uncompared where the scaled value is NaN (the oracle's cast of NaN to an integer is undefined in C++)."""
+    assert equal_where_not_nan(got["residual_out"], want["residual_out"]), "residual_out"
+    assert equal_where_not_nan(got["norm_out"], want["norm_out"]), "norm_out"
+    if quant == "none":
+        return
+    if quant != "fp8_static":
+        assert equal_where_not_nan(got["scale"].reshape(-1), want["scale"].reshape(-1)), "scales"
+    if quant == "int8_token":
+        y = want["norm_out"].float()
+        sc = want["scale"].reshape(-1, 1)
+        scaled_nan = torch.isnan(y / torch.where(sc > 0, sc, torch.ones_like(sc)))
+        assert equal_where_not_nan(got["q"], want["q"], ignore=scaled_nan), "int8 codes"
+    else:
+        assert equal_where_not_nan(got["q"], want["q"], nan_codes=True), "fp8 codes"
+
+
+@pytest.mark.parametrize("quant", ["none", "fp8_token", "fp8_group", "int8_token", "fp8_static"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("hidden,vpt", [(256, 0), (2048, 1), (8192, 4), (4096, 2)])
+def test_nonfinite_rows(cuda_device, dtype, quant, hidden, vpt):
+    """NaN, +inf and -inf in a partial, in the residual and in gamma: the eager composition (test/test_all_reduce_fusion.py:
+    23-28,75) is made of NaN-propagating torch ops, and so are amax and clamp in the quantizer.  A NaN anywhere in a row
+    makes the whole normed row NaN and its scale NaN; an infinity makes the reciprocal RMS zero, the infinite elements
+    NaN and the rest zero; gamma's NaN and infinities reach only their own columns (and their group's or row's scale).
+    The kernel's outputs must be the oracle's with NaN matching NaN."""
+    if dtype == torch.float32 and hidden > 4096:
+        hidden = 4096
+    p, r, g = eager.make_inputs(4, 12, hidden, dtype, 0.5, seed=401 + hidden)
+    last = hidden - 1
+    p[1, 0, 5] = float("nan")          # one NaN in the first wavefront's part of the row
+    p[2, 1, last - 3] = float("inf")   # +inf in the last wavefront's part
+    p[0, 2, hidden // 2] = float("-inf")
+    r[3, 11] = float("nan")
+    r[4, 3] = float("inf")
+    p[3, 5, 7] = float("inf")
+    p[1, 5, 7] = float("-inf")         # inf - inf in the reduction
+    p[0, 6, 130 % hidden] = float("inf")
+    r[6, 130 % hidden] = float("-inf")  # inf - inf in the residual add
+    # rows 7.. stay finite
+    for gamma_case in ("finite", "special"):
+        gamma = g.clone()
+        if gamma_case == "special":
+            gamma[100] = float("nan")
+            gamma[hidden - 126] = float("inf")
+            gamma[hidden - 60] = float("-inf")
+            gamma[17] = -1.0
+        static_scale = 0.0123 if quant == "fp8_static" else None
+        want = eager.reduce_rms(p, r, gamma, 1e-5, quant, static_scale=static_scale)
+        got = run_hip(p, r, gamma, 1e-5, quant, vecs_per_thread=vpt, static_scale=static_scale or 0.0)
+        _check_nonfinite(got, want, quant)
+        # the finite rows with finite gamma are ordinary rows: bit for bit, no NaN anywhere
+        if gamma_case == "finite":
+            assert not torch.isnan(got["norm_out"][7:].float()).any()
+            assert bits_equal(got["norm_out"][7:], want["norm_out"][7:])
+            assert torch.isnan(got["norm_out"][:7].float()).any(dim=1).all()
+
+
+@pytest.mark.parametrize("quant", ["fp8_token", "fp8_group", "int8_token", "fp8_static"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_negative_gamma_and_the_sign_of_zero(cuda_device, dtype, quant):
+    """Negative gamma on a zero element gives a normed -0, whose e4m3 code is 0x80, not 0x00: the quotient has to
+    keep the sign of a zero numerator.  Also rows that are zero throughout with mixed-sign gamma."""
+    p, r, g = eager.make_inputs(4, 9, 1024, dtype, 0.5, seed=77)
+    g[::3] = -g[::3]
+    p[:, :, 40:48] = 0.0
+    r[:, 40:48] = 0.0       # zero elements under both signs of gamma (columns 42 and 45 are negative)
+    p[:, 4] = 0.0
+    r[4] = 0.0              # an all-zero row: scale 0, codes +-0
+    static_scale = 0.05 if quant == "fp8_static" else None
+    want = eager.reduce_rms(p, r, g, 1e-5, quant, static_scale=static_scale)
+    got = run_hip(p, r, g, 1e-5, quant, static_scale=static_scale or 0.0)
+    assert bits_equal(got["norm_out"], want["norm_out"])
+    assert (want["norm_out"].view(torch.int16 if dtype != torch.float32 else torch.int32)[:, 42] < 0).any()   # a -0 is there
+    assert bits_equal(got["q"], want["q"]), "codes differ (sign of zero?)"
+    if quant != "fp8_static":
+        assert bits_equal(got["scale"].reshape(-1), want["scale"].reshape(-1))
+    if quant.startswith("fp8"):
+        assert (got["q"].view(torch.uint8) == 0x80).any()
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("scale", [1e-30, 3e-39, 1e-6, 1e4])
 def test_extreme_magnitudes(cuda_device, dtype, scale):
@@ -742,14 +830,35 @@ def test_doubles(cuda_device, n, tokens, hidden):
     _case("f64 table", p, r, g, 1e-6, "none", use_table=True, rank=1)
 
 
+@pytest.mark.parametrize("n,tokens,hidden", [(2, 33, 1024), (4, 129, 2048), (8, 7, 258), (4, 1000, 1536)])
+def test_doubles_through_the_staged_algorithms(cuda_device, n, tokens, hidden):
+    """The reference sends doubles through either of its kernels (src/ops/all_reduce_fusion.cpp:29-33,
+    all_reduce_fusion_impl.h:491): the two-launch structure for doubles -- all rows staged, this rank's rows staged
+    with the others delivered, and the N + 1 phase calls -- against the oracle, and bit-identical to the fused kernel."""
+    p, r, g = eager.make_inputs(n, tokens, hidden, torch.float64, 1.0, seed=650 + n)
+    fused, want, _ = _case("f64 fused", p, r, g, 1e-6, "none")
+    staged, _, _ = _case("f64 staged", p, r, g, 1e-6, "none", algo=_capi.ALGO_STAGED)
+    sums = torch.zeros((tokens, hidden), dtype=torch.float64)
+    for k in range(n):
+        sums = sums + p[k]
+    init = sums.clone()
+    init[1::n] = float("nan")
+    owned = run_hip(p, r, g, 1e-6, "none", algo=_capi.ALGO_STAGED_OWNED, rank=1, stage_init=init)
+    assert bits_equal(owned.pop("stage"), sums)
+    calls = [(("reduce",), k) for k in range(n)] + [(("norm",), 0)]
+    phased = run_hip(p, r, g, 1e-6, "none", algo=_capi.ALGO_STAGED_OWNED, calls=calls,
+                     stage_init=torch.full((tokens, hidden), float("nan"), dtype=torch.float64))
+    assert bits_equal(phased.pop("stage"), sums)
+    for other in (staged, owned, phased):
+        for k in fused:
+            assert bits_equal(fused[k], other[k]), k
+
+
 def test_doubles_limits(cuda_device):
     p, r, g = eager.make_inputs(2, 4, 256, torch.float64, 1.0, seed=1)
     with pytest.raises(_capi.TdeError) as ei:
         run_hip(p, r, g, 1e-6, "fp8_token")
     assert ei.value.status == _capi.EQUANT
-    with pytest.raises(_capi.TdeError) as ei:
-        run_hip(p, r, g, 1e-6, "none", algo=_capi.ALGO_STAGED)
-    assert ei.value.status == _capi.EALGO
     with pytest.raises(_capi.TdeError) as ei:
         run_hip(p, r, g, 1e-6, "none", calls=[(("traffic",), 0)])
     assert ei.value.status == _capi.EDTYPE

@@ -99,7 +99,7 @@ def test_error_paths_raise(tde, cuda_device):
     with pytest.raises(RuntimeError, match="not a pointer table handed out"):
         tde.allreduce_rms_fusion_impl(0, 2, x, x, g, torch.empty_like(x), torch.empty_like(x), 1e-6, ws.clone())
     y = torch.zeros((4, 8200), dtype=torch.bfloat16, device=cuda_device)
-    with pytest.raises(AssertionError):
+    with pytest.raises(RuntimeError, match="hidden_dim <= 8192"):   # the reference asserts (torch_dist_ext/__init__.py:68)
         tde.allreduce_rms(0, 2, y, y, torch.ones(8200, dtype=torch.bfloat16, device=cuda_device), 1e-6, ws)
 
 

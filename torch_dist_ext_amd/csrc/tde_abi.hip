@@ -67,25 +67,24 @@ constexpr int64_t kLoadsInFlightPerCu = 128 * 1024; // target for the limit on r
 constexpr int64_t kLimitFromWorkgroupsPerCu8 = 24, kLimitFromWorkgroupsPerCu4 = 32;
 constexpr int kDefaultComputeUnits = 256; // MI355X; used when no device can be asked (planning on a host without one)
 
-// Compute units of the current device, asked once per device.
+// Compute units of the current device, asked once per device and thread (no lock on the launch path).
 int compute_units() {
-    static std::mutex mu;
-    static int cached[kMaxDevices] = {};
+    thread_local int cached_dev = -1, cached_cu = 0;
     int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0) {
         (void)hipGetLastError();
         return kDefaultComputeUnits;
     }
-    std::lock_guard<std::mutex> lock(mu);
-    if (cached[dev] == 0) {
+    if (dev != cached_dev) {
         int cu = 0;
         if (hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cu <= 0) {
             (void)hipGetLastError();
             cu = kDefaultComputeUnits;
         }
-        cached[dev] = cu;
+        cached_dev = dev;
+        cached_cu = cu;
     }
-    return cached[dev];
+    return cached_cu;
 }
 
 int validate(const tde_problem *p, tde::Geometry *geo) {
@@ -101,10 +100,7 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     if (p->quant == TDE_QUANT_FP8_STATIC && !(p->static_scale > 0.0f && p->static_scale <= 3.0e38f)) return TDE_EQUANT;
     if (p->quant == TDE_QUANT_FP8_GROUP && p->hidden % TDE_QUANT_GROUP != 0) return TDE_EQUANT;
     if (p->algo < TDE_ALGO_AUTO || p->algo > TDE_ALGO_STAGED_OWNED) return TDE_EALGO;
-    if (p->dtype == TDE_F64) { // doubles: the fused kernel only, and no quantized output
-        if (p->quant != TDE_QUANT_NONE) return TDE_EQUANT;
-        if (p->algo == TDE_ALGO_STAGED || p->algo == TDE_ALGO_STAGED_OWNED) return TDE_EALGO;
-    }
+    if (p->dtype == TDE_F64 && p->quant != TDE_QUANT_NONE) return TDE_EQUANT; // doubles: no quantized output
     const int vec = 16 / eb;
     const int64_t nvec = p->hidden / vec;
     if (nvec > kMaxBlock) return TDE_EHIDDEN; // as the reference: one 16-byte vector per thread, 1024 threads
@@ -178,7 +174,12 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     if (geo) {
         geo->wgs_per_cu = wgs_per_cu;
         size_t lds = tde::sumsq_lds_bytes(tpr * rpb, vpt, vec);
-        if (wgs_per_cu > 0) lds = std::max(lds, tde::lds_bytes_for_workgroups_per_cu(wgs_per_cu)); // never with doubles
+        if (wgs_per_cu > 0) {
+            lds = std::max(lds, tde::lds_bytes_for_workgroups_per_cu(wgs_per_cu)); // never with doubles
+            // what the launch enforces: a geometry whose own LDS is larger than the padding admits fewer still
+            // (64: the kernels' static LDS)
+            geo->wgs_per_cu = (int)std::min<size_t>((size_t)wgs_per_cu, tde::kLdsPerCu / (lds + 64));
+        }
         geo->lds_bytes = (int)lds;
         geo->vec_elems = vec;
         geo->nvec = (int)nvec;
@@ -189,7 +190,7 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
         geo->grid = grid;
         // Row groups per XCD chunk of the row mapping (tde_rows.h: xcd_chunked_block); 16 measured best with 8
         // partials, 8 with 4.
-        geo->xcd_chunk = (p->dtype == TDE_F64) ? 1 : (p->nranks >= 8 ? 16 : 8);
+        geo->xcd_chunk = p->nranks >= 8 ? 16 : 8;
     }
     return TDE_OK;
 }
@@ -439,6 +440,7 @@ int run_phases(const tde_problem *p, const tde_buffers *b, void *hip_stream, int
         case TDE_BF16: e = tde::launch_reduce_bf16(n, a, span_bytes, first, step, rows, stream); break;
         case TDE_F16: e = tde::launch_reduce_f16(n, a, span_bytes, first, step, rows, stream); break;
         case TDE_F32: e = tde::launch_reduce_f32(n, a, span_bytes, first, step, rows, stream); break;
+        case TDE_F64: e = tde::launch_reduce_f64(n, a, span_bytes, first, step, rows, stream); break;
         }
         if (e != hipSuccess) return hip_fail(e);
     }

@@ -906,6 +906,7 @@ hipError_t launch_reduce_f32(int n, const RowArgs &a, int64_t row_bytes, int64_t
 
 // Rows of doubles (tde_rows_f64.hip): one vector per thread, no quantized output.
 hipError_t launch_rows_f64(int n, const RowArgs &a, const Geometry &g, hipStream_t s);
+hipError_t launch_reduce_f64(int n, const RowArgs &a, int64_t row_bytes, int64_t first_row, int64_t row_step, int64_t rows, hipStream_t s);
 
 // Traffic skeleton of the row kernel (tde_probe.hip): same geometry and bytes, no arithmetic.
 hipError_t launch_traffic(int n, int vpt, int code_bytes, bool wn, const RowArgs &a, const Geometry &g, uint32_t row_bytes,

@@ -4,7 +4,8 @@
 //   x   = ((0 + p_0) + ... + p_{N-1}) + residual_in        all in double, rank order          -> residual_out
 //   rs  = 1 / sqrt( sum(float(x)^2) / H + eps )             fp32: RMSNorm.forward squares x.float()
 //   y   = gamma * (x * double(rs))                          double                              -> norm_out
-// No quantized output for this type.  One 16-byte vector per thread, the row kernel's geometry.
+// No quantized output for this type.  One 16-byte vector per thread, the row kernel's geometry and XCD-aware row
+// mapping.  N == 0: the sum was staged (part[0] holds it), as in the row kernel; reduce_kernel_f64 is that stage A.
 #include <hip/hip_runtime.h>
 
 #include "tde_rows.h"
@@ -33,6 +34,7 @@ __device__ __forceinline__ u32x4 pack_f64(const double (&d)[2]) {
 
 template <int N>
 __global__ void __launch_bounds__(1024) row_kernel_f64(const RowArgs a) {
+    constexpr int NP = (N == 0) ? 1 : N;
     extern __shared__ __attribute__((aligned(16))) float lds_dyn[]; // squares (two per thread), then block sums
     float *const lds_img = lds_dyn;
     float *const lds_bs = lds_dyn + blockDim.x * 2;
@@ -44,12 +46,12 @@ __global__ void __launch_bounds__(1024) row_kernel_f64(const RowArgs a) {
     const uint32_t row_bytes = (uint32_t)a.hidden * 8u;
     const uint32_t off = (uint32_t)t * 16u;
 
-    const void *part[N];
+    const void *part[NP];
 #pragma unroll
-    for (int r = 0; r < N; ++r) part[r] = a.part[r];
+    for (int r = 0; r < NP; ++r) part[r] = a.part[r];
     if (a.table != nullptr) {
 #pragma unroll
-        for (int r = 0; r < N; ++r) {
+        for (int r = 0; r < NP; ++r) {
             const void *from_table = a.table[r];
             part[r] = (part[r] != nullptr) ? part[r] : from_table;
         }
@@ -57,23 +59,28 @@ __global__ void __launch_bounds__(1024) row_kernel_f64(const RowArgs a) {
     const rsrc_t gamma_rsrc = row_rsrc(a.gamma, 0, row_bytes);
 
     {
-        const int64_t row = (int64_t)blockIdx.x * a.rows_per_block + group; // the grid covers every row
+        // the grid covers every row; each XCD takes runs of consecutive row groups (xcd_chunked_block)
+        const int64_t row = (int64_t)xcd_chunked_block(blockIdx.x, gridDim.x, (uint32_t)a.xcd_chunk) * a.rows_per_block + group;
 
         const uint32_t bytes = (row < a.tokens) ? row_bytes : 0u;
         const int64_t row_byte = row * (int64_t)row_bytes;
-        u32x4 praw[N];
+        u32x4 praw[NP];
 #pragma unroll
-        for (int r = 0; r < N; ++r) praw[r] = rsrc_load16(row_rsrc(part[r], row_byte, bytes), off);
+        for (int r = 0; r < NP; ++r) praw[r] = rsrc_load16(row_rsrc(part[r], row_byte, bytes), off);
         const u32x4 rraw = rsrc_load16(row_rsrc(a.residual_in, row_byte, bytes), off);
         const u32x4 graw = __builtin_amdgcn_raw_buffer_load_b128(gamma_rsrc, (int)off, 0, kAuxDefault);
 
         double acc[2] = {0.0, 0.0};
+        if constexpr (N == 0) {
+            unpack_f64(praw[0], acc); // the staged sum
+        } else {
 #pragma unroll
-        for (int r = 0; r < N; ++r) {
-            double p[2];
-            unpack_f64(praw[r], p);
-            acc[0] += p[0];
-            acc[1] += p[1];
+            for (int r = 0; r < N; ++r) {
+                double p[2];
+                unpack_f64(praw[r], p);
+                acc[0] += p[0];
+                acc[1] += p[1];
+            }
         }
         double res[2], x[2];
         unpack_f64(rraw, res);
@@ -96,10 +103,71 @@ __global__ void __launch_bounds__(1024) row_kernel_f64(const RowArgs a) {
     }
 }
 
+// Stage A for doubles: the reduce kernel's spans (ReduceSpan), sums in double from +0 in rank order.
+template <int N, int U>
+__global__ void __launch_bounds__(256) reduce_kernel_f64(const RowArgs a, const ReduceSpan sp) {
+    constexpr uint32_t SPAN = 256u * U * 16u; // bytes per workgroup
+    const void *part[N];
+#pragma unroll
+    for (int r = 0; r < N; ++r) part[r] = a.part[r];
+    if (a.table != nullptr) {
+#pragma unroll
+        for (int r = 0; r < N; ++r) {
+            const void *from_table = a.table[r];
+            part[r] = (part[r] != nullptr) ? part[r] : from_table;
+        }
+    }
+    const int64_t bid = xcd_chunked_block(blockIdx.x, gridDim.x, sp.xcd_chunk);
+    const int64_t k = bid / sp.spans_per_row;
+    const int64_t in_row = (bid - k * sp.spans_per_row) * SPAN;
+    const int64_t base = (sp.first_row + k * sp.row_step) * sp.row_bytes + in_row;
+    const int64_t left = sp.row_bytes - in_row;
+    const uint32_t bytes = left < (int64_t)SPAN ? (uint32_t)left : SPAN;
+    u32x4 raw[U][N];
+#pragma unroll
+    for (int r = 0; r < N; ++r) {
+        const rsrc_t rs = row_rsrc(part[r], base, bytes);
+#pragma unroll
+        for (int u = 0; u < U; ++u) raw[u][r] = rsrc_load16(rs, (uint32_t)(u * 256 + threadIdx.x) * 16u);
+    }
+    const rsrc_t out = row_rsrc(a.stage_out, base, bytes);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        double acc[2] = {0.0, 0.0};
+#pragma unroll
+        for (int r = 0; r < N; ++r) {
+            double p[2];
+            unpack_f64(raw[u][r], p);
+            acc[0] += p[0];
+            acc[1] += p[1];
+        }
+        __builtin_amdgcn_raw_buffer_store_b128(pack_f64(acc), out, (int)((u * 256 + threadIdx.x) * 16), 0, kAuxDefault);
+    }
+}
+
+hipError_t launch_reduce_f64(int n, const RowArgs &a, int64_t row_bytes, int64_t first_row, int64_t row_step, int64_t rows,
+                             hipStream_t s) {
+    constexpr int U = 4;
+    constexpr int64_t span = 256 * U * 16;
+    ReduceSpan sp{row_bytes, first_row, row_step, (row_bytes + span - 1) / span, rows == 1 ? 16u : 1u};
+    const int64_t blocks = rows * sp.spans_per_row;
+    if (blocks <= 0) return hipSuccess;
+    if (blocks > 0x7fffffff) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)blocks), block(256);
+    switch (n) {
+    case 2: hipLaunchKernelGGL((reduce_kernel_f64<2, U>), grid, block, 0, s, a, sp); break;
+    case 4: hipLaunchKernelGGL((reduce_kernel_f64<4, U>), grid, block, 0, s, a, sp); break;
+    case 8: hipLaunchKernelGGL((reduce_kernel_f64<8, U>), grid, block, 0, s, a, sp); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 hipError_t launch_rows_f64(int n, const RowArgs &a, const Geometry &g, hipStream_t s) {
     const dim3 grid((unsigned)g.grid), block((unsigned)g.block_threads);
     const size_t lds = (size_t)g.lds_bytes; // sumsq_lds_bytes(g.block_threads, 1, 2): doubles are never limited per CU
     switch (n) {
+    case 0: hipLaunchKernelGGL((row_kernel_f64<0>), grid, block, lds, s, a); break;
     case 2: hipLaunchKernelGGL((row_kernel_f64<2>), grid, block, lds, s, a); break;
     case 4: hipLaunchKernelGGL((row_kernel_f64<4>), grid, block, lds, s, a); break;
     case 8: hipLaunchKernelGGL((row_kernel_f64<8>), grid, block, lds, s, a); break;

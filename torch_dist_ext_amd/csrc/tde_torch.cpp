@@ -15,6 +15,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <tuple>
 #include <unordered_map>
 #include <vector>
 
@@ -165,6 +166,11 @@ public:
         return alias(tde_workspace_stage(ws_, (int32_t)rank_), ref);
     }
 
+    // Makes this workspace the one torch_dist_ext::get_workspace hands out (the reference keeps it in the Python
+    // package's global `comm`, torch_dist_ext/__init__.py:37-46; the operator is registered in C++ here, so the
+    // current workspace is kept here as well).  The previous one is released.
+    void make_current();
+
     int64_t rank() const { return rank_; }
     int64_t world_size() const { return world_size_; }
     int64_t size_in_bytes() const { return size_in_bytes_; }
@@ -185,6 +191,31 @@ private:
 };
 
 namespace {
+
+std::mutex g_current_mutex;
+// Never destroyed: releasing device memory during static destruction would run after the HIP runtime has gone.
+c10::intrusive_ptr<CommWorkspace> *g_current = new c10::intrusive_ptr<CommWorkspace>();
+
+} // namespace
+
+void CommWorkspace::make_current() {
+    auto self = c10::intrusive_ptr<CommWorkspace>::unsafe_reclaim_from_nonowning(this);
+    const std::lock_guard<std::mutex> lock(g_current_mutex);
+    *g_current = std::move(self);
+}
+
+namespace {
+
+// torch_dist_ext::get_workspace (reference: a Python custom_op over the package's global, torch_dist_ext/__init__.py:49-53).
+Tensor get_workspace_op(const Tensor &ref) {
+    c10::intrusive_ptr<CommWorkspace> cur;
+    {
+        const std::lock_guard<std::mutex> lock(g_current_mutex);
+        cur = *g_current;
+    }
+    TORCH_CHECK(cur.defined(), "torch_dist_ext::get_workspace: setup_env has not been called");
+    return cur->get_workspace(ref);
+}
 
 struct Call {
     tde_problem p{};
@@ -292,6 +323,75 @@ void allreduce_rms_quant_fusion(int64_t rank, int64_t nranks, Tensor &allreduce_
     run(c, allreduce_in);
 }
 
+// Functional form, the operator the reference's package defines in Python (torch_dist_ext/__init__.py:64-73:
+// a torch.library.custom_op that allocates norm_out and residual_out and calls allreduce_rms_fusion).  Registered
+// here instead, same name and schema: a Python custom_op costs 12 us of host time per call, which is more than
+// the kernel takes at decode sizes.  The hidden_dim <= 8192 assertion of the reference (:68) is a check here.
+std::tuple<Tensor, Tensor> allreduce_rms(int64_t rank, int64_t nranks, const Tensor &allreduce_in, const Tensor &residual_in,
+                                         const Tensor &rms_gamma, double eps, const Tensor &workspace) {
+    TORCH_CHECK(allreduce_in.dim() >= 1 && allreduce_in.size(-1) <= 8192, "allreduce_rms: hidden_dim <= 8192 expected");
+    Tensor norm_out = at::empty_like(allreduce_in);
+    Tensor residual_out = at::empty_like(residual_in);
+    Call c;
+    fill_common(c, rank, nranks, allreduce_in, residual_in, rms_gamma, residual_out, eps);
+    c.p.quant = TDE_QUANT_NONE;
+    c.b.norm_out = norm_out.data_ptr();
+    c.p.write_norm = 1;
+    use_table(c, rank, nranks, allreduce_in, workspace);
+    run(c, allreduce_in);
+    return {norm_out, residual_out};
+}
+
+// Shapes and dtypes only: what tracing (fake tensors, torch.compile) sees.
+std::tuple<Tensor, Tensor> allreduce_rms_meta(int64_t, int64_t, const Tensor &allreduce_in, const Tensor &residual_in,
+                                              const Tensor &, double, const Tensor &) {
+    return {at::empty_like(allreduce_in), at::empty_like(residual_in)};
+}
+
+struct QuantOutputs {
+    Tensor q, scale, residual_out, norm_out;
+};
+
+// Output tensors of the quantizing operator: codes (e4m3 or int8) shaped like the input, scales [..., 1] per row or
+// [..., hidden/128] per group (no elements with a static scale), residual_out, and norm_out (no elements unless asked for).
+QuantOutputs quant_outputs(const Tensor &allreduce_in, const Tensor &residual_in, int64_t quant_mode, bool write_norm) {
+    TORCH_CHECK(allreduce_in.dim() >= 1 && allreduce_in.size(-1) <= 8192, "allreduce_rms_quant: hidden_dim <= 8192 expected");
+    TORCH_CHECK(quant_mode == TDE_QUANT_FP8_TOKEN || quant_mode == TDE_QUANT_FP8_GROUP || quant_mode == TDE_QUANT_INT8_TOKEN ||
+                    quant_mode == TDE_QUANT_FP8_STATIC,
+                "allreduce_rms_quant: quant_mode must be one of the quantizing modes (1..4)");
+    QuantOutputs o;
+    const auto q_dtype = quant_mode == TDE_QUANT_INT8_TOKEN ? at::kChar : at::kFloat8_e4m3fn;
+    o.q = at::empty(allreduce_in.sizes(), allreduce_in.options().dtype(q_dtype));
+    std::vector<int64_t> scale_shape(allreduce_in.sizes().begin(), allreduce_in.sizes().end() - 1);
+    if (quant_mode == TDE_QUANT_FP8_GROUP) scale_shape.push_back(allreduce_in.size(-1) / TDE_QUANT_GROUP);
+    if (quant_mode == TDE_QUANT_FP8_STATIC) scale_shape.assign(1, 0);
+    o.scale = at::empty(scale_shape, allreduce_in.options().dtype(at::kFloat));
+    o.residual_out = at::empty_like(residual_in);
+    o.norm_out = write_norm ? at::empty_like(allreduce_in) : at::empty({0}, allreduce_in.options());
+    return o;
+}
+
+std::tuple<Tensor, Tensor, Tensor, Tensor> allreduce_rms_quant(int64_t rank, int64_t nranks, const Tensor &allreduce_in,
+                                                               const Tensor &residual_in, const Tensor &rms_gamma, double eps,
+                                                               const Tensor &workspace, int64_t quant_mode, bool write_norm,
+                                                               double static_scale) {
+    QuantOutputs o = quant_outputs(allreduce_in, residual_in, quant_mode, write_norm);
+    Call c;
+    fill_common(c, rank, nranks, allreduce_in, residual_in, rms_gamma, o.residual_out, eps);
+    fill_quant(c, quant_mode, allreduce_in, write_norm ? c10::optional<Tensor>(o.norm_out) : c10::nullopt, o.q,
+               quant_mode == TDE_QUANT_FP8_STATIC ? c10::nullopt : c10::optional<Tensor>(o.scale), static_scale);
+    use_table(c, rank, nranks, allreduce_in, workspace);
+    run(c, allreduce_in);
+    return {o.q, o.scale, o.residual_out, o.norm_out};
+}
+
+std::tuple<Tensor, Tensor, Tensor, Tensor> allreduce_rms_quant_meta(int64_t, int64_t, const Tensor &allreduce_in,
+                                                                    const Tensor &residual_in, const Tensor &, double, const Tensor &,
+                                                                    int64_t quant_mode, bool write_norm, double) {
+    QuantOutputs o = quant_outputs(allreduce_in, residual_in, quant_mode, write_norm);
+    return {o.q, o.scale, o.residual_out, o.norm_out};
+}
+
 // The same stage with the N partials given directly as N tensors (no workspace object).
 void reduce_rms_local(std::vector<Tensor> partials, Tensor &residual_in, Tensor &rms_gamma, Tensor &residual_out,
                       c10::optional<Tensor> norm_out, c10::optional<Tensor> q_out, c10::optional<Tensor> scale_out,
@@ -323,6 +423,7 @@ TORCH_LIBRARY(torch_dist_ext, m) {
         .def("peer_partial", &CommWorkspace::peer_partial)
         .def("set_peer_partial", &CommWorkspace::set_peer_partial)
         .def("stage", &CommWorkspace::stage)
+        .def("make_current", &CommWorkspace::make_current)
         .def("rank", &CommWorkspace::rank)
         .def("world_size", &CommWorkspace::world_size)
         .def("size_in_bytes", &CommWorkspace::size_in_bytes);
@@ -331,6 +432,11 @@ TORCH_LIBRARY(torch_dist_ext, m) {
     m.def("allreduce_rms_quant_fusion(SymInt rank, SymInt nranks, Tensor allreduce_in, Tensor residual_in, Tensor rms_gamma, "
           "Tensor residual_out, Tensor? norm_out, Tensor q_out, Tensor? scale_out, float eps, Tensor workspace, "
           "int quant_mode, float static_scale=0.0) -> ()");
+    m.def("get_workspace(Tensor ref) -> Tensor");
+    m.def("allreduce_rms(SymInt rank, SymInt nranks, Tensor allreduce_in, Tensor residual_in, Tensor rms_gamma, float eps, "
+          "Tensor workspace) -> (Tensor, Tensor)");
+    m.def("allreduce_rms_quant(SymInt rank, SymInt nranks, Tensor allreduce_in, Tensor residual_in, Tensor rms_gamma, float eps, "
+          "Tensor workspace, SymInt quant_mode, bool write_norm, float static_scale=0.0) -> (Tensor, Tensor, Tensor, Tensor)");
     m.def("reduce_rms_local(Tensor[] partials, Tensor residual_in, Tensor rms_gamma, Tensor residual_out, "
           "Tensor? norm_out, Tensor? q_out, Tensor? scale_out, float eps, int quant_mode, int algo, Tensor? stage, "
           "float static_scale=0.0) -> ()");
@@ -340,4 +446,12 @@ TORCH_LIBRARY_IMPL(torch_dist_ext, CUDA, m) {
     m.impl("allreduce_rms_fusion", &allreduce_rms_fusion);
     m.impl("allreduce_rms_quant_fusion", &allreduce_rms_quant_fusion);
     m.impl("reduce_rms_local", &reduce_rms_local);
+    m.impl("allreduce_rms", &allreduce_rms);
+    m.impl("allreduce_rms_quant", &allreduce_rms_quant);
+    m.impl("get_workspace", &get_workspace_op);
+}
+
+TORCH_LIBRARY_IMPL(torch_dist_ext, Meta, m) {
+    m.impl("allreduce_rms", &allreduce_rms_meta);
+    m.impl("allreduce_rms_quant", &allreduce_rms_quant_meta);
 }
