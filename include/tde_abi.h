@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define TDE_ABI_VERSION 3
+#define TDE_ABI_VERSION 4
 #define TDE_MAX_RANKS 16 /* array bound, as MAX_RANKS in src/ops/all_reduce_fusion.h:8 */
 #define TDE_QUANT_GROUP 128
 #define TDE_STATIC_STAGE_BYTES (32 << 20) /* stage held inside the library for tde_reduce_rms_static_stage */
@@ -180,9 +180,12 @@ int tde_stage_norm(const tde_problem *problem, const tde_buffers *buffers, void 
    HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
    reference, whose stage lives in the CommWorkspace allocation (src/ops/all_reduce_fusion.cpp:70-74).
    Limit: tokens * hidden * elem_size <= TDE_STATIC_STAGE_BYTES (32 MiB, e.g. 2048 x 8192 bf16), else
-   TDE_ETOOBIG.  Every GPU the library runs on holds one copy of the array until the process ends, and every
-   call on a GPU uses that copy: calls that overlap on one GPU (different streams, different threads) race.
-   Each call overwrites the part of the array it reads, so nothing needs clearing between calls. */
+   TDE_ETOOBIG.  Every GPU the library runs on holds one copy of the array until the process ends -- 32 MiB of
+   device memory per GPU for every process that loads the library, whether it calls this entry point or not -- and
+   every call on a GPU uses that copy: calls that overlap on one GPU (different streams, different threads) race,
+   silently; the library keeps no record of the streams it was given and cannot tell.
+   Each call overwrites the part of the array it reads, so nothing needs clearing between calls.
+   Note the meaning of TDE_ALGO_AUTO: the staged algorithm here, the fused one in tde_reduce_rms. */
 int tde_reduce_rms_static_stage(const tde_problem *problem, const tde_buffers *buffers, void *hip_stream);
 
 /* Calibration: enqueue a plain copy of `bytes` (multiple of 16) from src to dst on `hip_stream`.
@@ -235,7 +238,10 @@ int tde_device_info(tde_device_info_out *out);
    (comm_bufs[r] + size, impl.h:375,387). */
 typedef struct tde_workspace tde_workspace;
 
-int tde_workspace_create(int32_t nranks, int64_t slot_bytes, tde_workspace **out);
+/* nblocks: workgroups the reference's kernels would synchronize (1..65536; its package passes 256,
+   torch_dist_ext/__init__.py:24); it sizes the per-rank flag regions of the pointer table exactly as the reference
+   does, nblocks * nranks ints each (src/ops/all_reduce_fusion.cpp:72).  No kernel of this library reads the flags. */
+int tde_workspace_create(int32_t nranks, int32_t nblocks, int64_t slot_bytes, tde_workspace **out);
 int tde_workspace_destroy(tde_workspace *ws);
 /* Device pointer of slot r (first half). */
 void *tde_workspace_slot(const tde_workspace *ws, int32_t r);

@@ -8,7 +8,8 @@
 // linked as a checker only; residual_out is additionally required to be bit-exact against the
 // oracle's rank-order restatement.
 //
-// Build: python torch_dist_ext_amd/_build.py   (produces tests/native/unit_test_abi)
+// Build: python tests/native/build_native.py   (produces tests/native/unit_test_abi; links libtde_hip.so, built before
+//        it by python torch_dist_ext_amd/_build.py)
 // Run:   tests/native/unit_test_abi            (exit code 0 = every case validated)
 #include <hip/hip_runtime.h>
 

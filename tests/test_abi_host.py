@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), name
     assert sorted(_capi.EXPORTS) == declared
-    assert _capi.load().tde_abi_version() == _capi.ABI_VERSION == 3
+    assert _capi.load().tde_abi_version() == _capi.ABI_VERSION == 4
 
 
 def test_struct_layouts_match_header():
@@ -147,9 +147,10 @@ def test_reduce_rms_argument_checks_need_no_gpu():
 def test_workspace_argument_checks_need_no_gpu():
     lib = _capi.load()
     ws = ctypes.c_void_p()
-    assert lib.tde_workspace_create(3, 1024, ctypes.byref(ws)) == _capi.ENRANKS
-    assert lib.tde_workspace_create(2, 1000, ctypes.byref(ws)) == _capi.ESHAPE
-    assert lib.tde_workspace_create(2, 1024, None) == _capi.EINVAL
+    assert lib.tde_workspace_create(3, 256, 1024, ctypes.byref(ws)) == _capi.ENRANKS
+    assert lib.tde_workspace_create(2, 256, 1000, ctypes.byref(ws)) == _capi.ESHAPE
+    assert lib.tde_workspace_create(2, 256, 1024, None) == _capi.EINVAL
+    assert lib.tde_workspace_create(2, 0, 1024, ctypes.byref(ws)) == _capi.EINVAL      # nblocks sizes the flag regions
     assert lib.tde_workspace_destroy(None) == _capi.OK
     assert lib.tde_workspace_slot(None, 0) is None
 

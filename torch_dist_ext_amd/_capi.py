@@ -17,7 +17,7 @@ QUANT_NONE, QUANT_FP8_TOKEN, QUANT_FP8_GROUP, QUANT_INT8_TOKEN, QUANT_FP8_STATIC
 ALGO_AUTO, ALGO_FUSED, ALGO_STAGED, ALGO_STAGED_OWNED = 0, 1, 2, 3
 
 # Every symbol include/tde_abi.h declares.
-ABI_VERSION = 3   # TDE_ABI_VERSION of include/tde_abi.h
+ABI_VERSION = 4   # TDE_ABI_VERSION of include/tde_abi.h
 
 EXPORTS = (
     "tde_abi_version", "tde_status_string", "tde_last_hip_error", "tde_plan", "tde_reduce_rms", "tde_stage_reduce", "tde_stage_norm",
@@ -105,7 +105,7 @@ def load():
     lib.tde_device_info.restype = ctypes.c_int
     lib.tde_device_info.argtypes = [ctypes.POINTER(DeviceInfo)]
     lib.tde_workspace_create.restype = ctypes.c_int
-    lib.tde_workspace_create.argtypes = [ctypes.c_int32, ctypes.c_int64, ctypes.POINTER(ctypes.c_void_p)]
+    lib.tde_workspace_create.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int64, ctypes.POINTER(ctypes.c_void_p)]
     lib.tde_workspace_destroy.restype = ctypes.c_int
     lib.tde_workspace_destroy.argtypes = [ctypes.c_void_p]
     lib.tde_workspace_slot.restype = ctypes.c_void_p

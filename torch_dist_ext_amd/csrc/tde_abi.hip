@@ -249,9 +249,10 @@ __global__ void __launch_bounds__(256) stream_kernel(const void *src, void *dst,
 
 struct tde_workspace {
     int32_t nranks;
+    int32_t nblocks;
     int64_t slot_bytes;
     void *slots[TDE_MAX_RANKS];
-    void *flags;   // nranks regions of 256*nranks ints, zeroed (layout parity only)
+    void *flags;   // nranks regions of nblocks*nranks ints, zeroed (layout parity only: no kernel here reads them)
     int32_t *cells; // 5 int cells: counter, two-shot clock, one-shot clock, one-shot size, one-shot clear
 };
 
@@ -502,18 +503,21 @@ int tde_probe_rows_parts(const tde_problem *p, const tde_buffers *b, int32_t par
 
 // ---- emulated peer workspace ----------------------------------------------------------------
 
-int tde_workspace_create(int32_t nranks, int64_t slot_bytes, tde_workspace **out) {
+int tde_workspace_create(int32_t nranks, int32_t nblocks, int64_t slot_bytes, tde_workspace **out) {
     if (out == nullptr) return TDE_EINVAL;
     *out = nullptr;
     if (!(nranks == 2 || nranks == 4 || nranks == 8)) return TDE_ENRANKS;
+    if (nblocks < 1 || nblocks > 65536) return TDE_EINVAL;
     if (slot_bytes <= 0 || slot_bytes % 16 != 0) return TDE_ESHAPE;
     tde_workspace *ws = new (std::nothrow) tde_workspace();
     if (ws == nullptr) return TDE_ENOMEM;
     ws->nranks = nranks;
+    ws->nblocks = nblocks;
     ws->slot_bytes = slot_bytes;
     hipError_t e = hipSuccess;
     for (int r = 0; r < nranks && e == hipSuccess; ++r) e = hipMalloc(&ws->slots[r], (size_t)slot_bytes * 2);
-    const size_t flag_bytes = (size_t)nranks * 256 * nranks * sizeof(int32_t);
+    // one flag region per rank, each nblocks * nranks ints as the reference sizes it (src/ops/all_reduce_fusion.cpp:72)
+    const size_t flag_bytes = (size_t)nranks * nblocks * nranks * sizeof(int32_t);
     if (e == hipSuccess) e = hipMalloc(&ws->flags, flag_bytes);
     if (e == hipSuccess) e = hipMemset(ws->flags, 0, flag_bytes);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ws->cells), 5 * 64);
@@ -557,7 +561,7 @@ int tde_workspace_fill_table(const tde_workspace *ws, void **table, int32_t entr
     if (entries != 3 * n + 5) return TDE_EINVAL;
     for (int r = 0; r < n; ++r) {
         table[r] = ws->slots[r];
-        table[n + r] = static_cast<char *>(ws->flags) + (size_t)r * 256 * n * sizeof(int32_t);
+        table[n + r] = static_cast<char *>(ws->flags) + (size_t)r * ws->nblocks * n * sizeof(int32_t);
         table[2 * n + r] = ws->slots[r];
     }
     for (int c = 0; c < 5; ++c) table[3 * n + c] = reinterpret_cast<char *>(ws->cells) + 64 * c;

@@ -89,7 +89,8 @@ public:
         TORCH_CHECK(rank >= 0 && rank < world_size, "CommWorkspace: rank ", rank, " outside [0, ", world_size, ")");
         TORCH_CHECK(size_in_bytes > 0 && size_in_bytes % 16 == 0, "CommWorkspace: size_in_bytes must be a positive multiple of 16");
         device_ = c10::hip::current_device();
-        check_status(tde_workspace_create((int32_t)world_size, size_in_bytes, &ws_), "CommWorkspace");
+        TORCH_CHECK(nblocks >= 1 && nblocks <= 65536, "CommWorkspace: nblocks must be in [1, 65536]");
+        check_status(tde_workspace_create((int32_t)world_size, (int32_t)nblocks, size_in_bytes, &ws_), "CommWorkspace");
     }
 
     ~CommWorkspace() override {
