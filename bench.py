@@ -39,8 +39,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 # They describe the kernels whose sources hash to `sources_sha256`; with any other kernel source the bench line reports
 # traffic as null.
 TRAFFIC = {
-    "sources_sha256": "83fc4b01bcba134fe66bbedb518b7eb987f60f614962844edf2984a0b67b1734",
-    "bytes": {"c2": 11694347, "c3": 352654238, "c4": 765471037, "c5": 2181253551},
+    "sources_sha256": "cb36b78742d24dbc6f8aed6b42621d47f975a3eab81bb4b562febaea200f20fe",
+    "bytes": {"c2": 11697298, "c3": 352648337, "c4": 765465820, "c5": 2181241993},
 }
 
 BENCH_CONFIGS = {
@@ -212,7 +212,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fit", action="store_true", help="skip roofline.fit (the same kernel at three row counts)")
     ap.add_argument("--operator-path", action="store_true",
-                    help="also time the torch operator path on one set of buffers (always done for c2)")
+                    help="also time the torch operator path on one set of buffers (done for c2 unless --no-operator-path)")
+    ap.add_argument("--no-operator-path", action="store_true")
     ap.add_argument("--algo", default="auto", choices=["auto", "fused", "staged", "staged_owned"])
     ap.add_argument("--settle-ms", type=float, default=20.0,
                     help="before the warm-up steps, run the same step untimed for about this long (0 = not at all; steps shorter "
@@ -391,41 +392,6 @@ def main():
         kernel_out["q"] = s0["q"].cpu()
         kernel_out["scale"] = s0["scale"].cpu()
 
-    # The same kernel at three row counts, in blocks of the same rotating buffers (or of larger ones), and the
-    # straight line through the three points: time = fixed_us + bytes / bulk_GBs.
-    fit = None
-    if not args.no_fit and not staged and T >= 4:
-        grow = (N + 2) * 4 * T * H * e <= (2 << 30)     # sets of 4 T rows stay below 2 GiB each: fit at T, 2T, 4T
-        rows_list = [T, 2 * T, 4 * T] if grow else [T // 4, T // 2, T]
-        top = rows_list[-1]
-        if grow:
-            fit_sets = make_sets(torch, cfg, max(3, -(-(5 << 30) // ((N + 2) * top * H * e))), dev, None, rows=top)
-        else:
-            fit_sets = sets
-        points = []
-        for rows in rows_list:
-            blocks = argument_blocks(fit_sets, top, rows)
-            refs = [ctypes.byref(b) for b in blocks]
-            p_rows = problem(rows)
-            pr = ctypes.byref(p_rows)
-
-            def launch_rows(i, pr=pr, refs=refs):
-                st = lib.tde_reduce_rms(pr, refs[i % len(refs)], hip_stream)
-                if st != 0:
-                    _capi.check(st)
-            steps = max(20, min(args.steps, int(args.steps * T / rows)))
-            points.append((rows, _capi.plan(p_rows).algorithmic_bytes, timed(launch_rows, steps, args.warmup)))
-        n = len(points)
-        mx = sum(p[1] for p in points) / n
-        my = sum(p[2] for p in points) / n
-        slope = sum((p[1] - mx) * (p[2] - my) for p in points) / sum((p[1] - mx) ** 2 for p in points)   # us per byte
-        fit = {"rows": [p[0] for p in points], "kernel_us": [p[2] for p in points],
-               "frac_of_peak": [p[1] / (p[2] * 1e-6) / 1e9 / HBM_PEAK_GBS for p in points],
-               "fixed_us": my - slope * mx, "bulk_GBs": 1e-3 / slope}
-        if grow:
-            del fit_sets
-            torch.cuda.empty_cache()
-
     # The same launches with the arithmetic removed (tde_probe_rows_parts): what the access pattern alone takes
     # on this box, in this process, over the same buffers -- all of it, its input streams alone, its output
     # streams alone.  They overwrite the outputs, hence after the timed run.
@@ -440,6 +406,31 @@ def main():
                 if st != 0:
                     _capi.check(st)
             pattern[key] = timed(launch_parts, args.steps, args.warmup)
+    if "reads_only_us" in pattern and "writes_only_us" in pattern:
+        # The input streams and the output streams as two kernels at once, on two streams: different workgroups on
+        # different compute units, the same memory system.  Against traffic_only_us (both in one kernel) this tells
+        # whether mixing reads with writes costs on the compute units or behind them.  The span is taken on the launch
+        # stream, which waits for both side streams; the cross-stream waits cost about a microsecond per step.
+        side = [torch.cuda.Stream(dev), torch.cuda.Stream(dev)]
+        side_h = [ctypes.c_void_p(x.cuda_stream) for x in side]
+
+        def both_at_once(steps):
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            done = [torch.cuda.Event(), torch.cuda.Event()]
+            begin.record(stream)
+            for x in side:
+                x.wait_event(begin)
+            for i in range(steps):
+                lib.tde_probe_rows_parts(prob_ref, call_refs[i % nsets], 1, side_h[0])
+                lib.tde_probe_rows_parts(prob_ref, call_refs[i % nsets], 6, side_h[1])
+            for x, ev in zip(side, done):
+                ev.record(x)
+                stream.wait_event(ev)
+            end.record(stream)
+            torch.cuda.synchronize(dev)
+            return begin.elapsed_time(end) * 1e3 / steps
+        both_at_once(args.warmup)
+        pattern["reads_and_writes_as_two_concurrent_kernels_us"] = both_at_once(args.steps)
     floor_us = pattern.get("traffic_only_us")
     read_bytes = (N + 1) * T * H * e
     launch_floor_us = timed(lambda i: lib.tde_probe_launch(hip_stream), 500, 50)
@@ -477,7 +468,7 @@ def main():
                      # W warm-up + K launches timed the same way before the settling phase (a device that has just been idle)
                      "cold_kernel_avg_us": cold_avg_us,
                      "cold_frac": bytes_per_launch / (cold_avg_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
-                     "fit": fit,
+                     "fit": None,   # filled in below
                      # the same launches without arithmetic (same bytes, same access pattern), and their share of the peak
                      "traffic_only_us": floor_us,
                      "traffic_only_frac": (bytes_per_launch / (floor_us * 1e-6) / 1e9 / HBM_PEAK_GBS) if floor_us else None,
@@ -486,15 +477,16 @@ def main():
                      "reads_only_GBs": (read_bytes / (pattern["reads_only_us"] * 1e-6) / 1e9) if pattern.get("reads_only_us") else None,
                      "writes_only_us": pattern.get("writes_only_us"),
                      "writes_only_GBs": (out_bytes / (pattern["writes_only_us"] * 1e-6) / 1e9) if pattern.get("writes_only_us") else None,
+                     "reads_and_writes_as_two_concurrent_kernels_us": pattern.get("reads_and_writes_as_two_concurrent_kernels_us"),
                      # one empty dispatch, back to back on the same stream: the floor under latency-bound sizes
                      "launch_floor_us": launch_floor_us},
     }
     # The device's practical streaming rates, measured now (tde_probe_stream: 1 GiB per launch, four buffers
     # in rotation): what reads alone, writes alone and a plain copy reach on this box.
-    del sets, calls, call_refs
-    torch.cuda.empty_cache()
-    if args.operator_path or args.config == "c2":
-        out["operator_path"] = operator_path_cost(torch, cfg, first, dev)
+    # Nothing has been given back to the driver so far, and nothing is until every rate is measured: after device
+    # memory is freed (torch.cuda.empty_cache -> hipFree) memory-bound launches run about 1.4 % slower for some
+    # hundred milliseconds (c3: kernel 57.2 -> 58.0 us, skeleton 55.8 -> 56.6, measured by freeing 7 GiB between two
+    # timings), presumably the driver clearing the freed pages in the background.
     gib = 1 << 30
     bufs = [torch.empty(gib, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(4)]
     rates = {}
@@ -503,6 +495,44 @@ def main():
                                                            stream.cuda_stream), 12, 3)
         rates[name] = moved / (us * 1e-6) / 1e9
     del bufs
+
+    # The same kernel at three row counts, in blocks of the same rotating buffers (or of larger ones), and the
+    # straight line through the three points: time = fixed_us + bytes / bulk_GBs.
+    fit = None
+    if not args.no_fit and not staged and T >= 4:
+        grow = (N + 2) * 4 * T * H * e <= (2 << 30)     # sets of 4 T rows stay below 2 GiB each: fit at T, 2T, 4T
+        rows_list = [T, 2 * T, 4 * T] if grow else [T // 4, T // 2, T]
+        top = rows_list[-1]
+        if grow:
+            fit_sets = make_sets(torch, cfg, max(3, -(-(5 << 30) // ((N + 2) * top * H * e))), dev, None, rows=top)
+        else:
+            fit_sets = sets
+        points = []
+        for rows in rows_list:
+            blocks = argument_blocks(fit_sets, top, rows)
+            refs = [ctypes.byref(b) for b in blocks]
+            p_rows = problem(rows)
+            pr = ctypes.byref(p_rows)
+
+            def launch_rows(i, pr=pr, refs=refs):
+                st = lib.tde_reduce_rms(pr, refs[i % len(refs)], hip_stream)
+                if st != 0:
+                    _capi.check(st)
+            steps = max(20, min(args.steps, int(args.steps * T / rows)))
+            points.append((rows, _capi.plan(p_rows).algorithmic_bytes, timed(launch_rows, steps, args.warmup)))
+        n = len(points)
+        mx = sum(p[1] for p in points) / n
+        my = sum(p[2] for p in points) / n
+        slope = sum((p[1] - mx) * (p[2] - my) for p in points) / sum((p[1] - mx) ** 2 for p in points)   # us per byte
+        fit = {"rows": [p[0] for p in points], "kernel_us": [p[2] for p in points],
+               "frac_of_peak": [p[1] / (p[2] * 1e-6) / 1e9 / HBM_PEAK_GBS for p in points],
+               "fixed_us": my - slope * mx, "bulk_GBs": 1e-3 / slope}
+        if grow:
+            del fit_sets   # back to torch's allocator, not to the driver
+
+    out["roofline"]["fit"] = fit
+    if args.operator_path or (args.config == "c2" and not args.no_operator_path):
+        out["operator_path"] = operator_path_cost(torch, cfg, first, dev)
     info = _capi.device_info()
     out["device"] = {"name": torch.cuda.get_device_properties(dev).name, "compute_units": info.compute_units,
                      "memory_clock_khz": info.memory_clock_khz, "memory_bus_bits": info.memory_bus_bits,
