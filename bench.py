@@ -40,7 +40,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 # traffic as null.
 TRAFFIC = {
     "sources_sha256": "cb36b78742d24dbc6f8aed6b42621d47f975a3eab81bb4b562febaea200f20fe",
-    "bytes": {"c2": 11697298, "c3": 352648337, "c4": 765465820, "c5": 2181241993},
+    "bytes": {"c2": 11696832, "c3": 352648977, "c4": 765464707, "c5": 2181272138},
 }
 
 BENCH_CONFIGS = {
@@ -429,7 +429,8 @@ def main():
             end.record(stream)
             torch.cuda.synchronize(dev)
             return begin.elapsed_time(end) * 1e3 / steps
-        both_at_once(args.warmup)
+        if args.warmup > 0:
+            both_at_once(args.warmup)
         pattern["reads_and_writes_as_two_concurrent_kernels_us"] = both_at_once(args.steps)
     floor_us = pattern.get("traffic_only_us")
     read_bytes = (N + 1) * T * H * e
