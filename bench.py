@@ -527,7 +527,9 @@ def main():
         slope = sum((p[1] - mx) * (p[2] - my) for p in points) / sum((p[1] - mx) ** 2 for p in points)   # us per byte
         fit = {"rows": [p[0] for p in points], "kernel_us": [p[2] for p in points],
                "frac_of_peak": [p[1] / (p[2] * 1e-6) / 1e9 / HBM_PEAK_GBS for p in points],
-               "fixed_us": my - slope * mx, "bulk_GBs": 1e-3 / slope}
+               "fixed_us": my - slope * mx,
+               # launch-bound sizes do not grow with the bytes: no rate to quote
+               "bulk_GBs": (1e-3 / slope) if slope > 0 else None}
         if grow:
             del fit_sets   # back to torch's allocator, not to the driver
 
