@@ -17,6 +17,7 @@ CASES = [
     # first call fills most of the 32 MiB array, the second reuses its beginning with other contents
     (8, 1536, 8192, torch.bfloat16, 0.5, 1e-5, "fp8_token", 21),
     (4, 37, 1024, torch.float16, 1.0, 1e-6, "int8_token", 22),
+    (2, 19, 2048, torch.float64, 1.0, 1e-6, "none", 24),      # doubles go through the staged launches as well
 ]
 
 
