@@ -309,7 +309,7 @@ int tdo_reduce_rms(int dtype, int nranks, int64_t tokens, int64_t hidden, const 
             float amax = 0.0f;
             for (int64_t h = g * group; h < (g + 1) * group; ++h) {
                 float a = fabsf(y[h]);
-                if (a > amax) amax = a;
+                if (a > amax || a != a) amax = a; /* a NaN stays: torch's amax propagates it (no later `>` replaces it) */
             }
             float scale = amax / qmax;
             scale_out[t * ngroups + g] = scale;

@@ -209,6 +209,39 @@ def test_c_restatement_in_torch_sum_order_is_bit_identical_to_eager(dtype, code,
         assert np.array_equal(c["q"], want["q"].view(torch.uint8).numpy())
 
 
+@pytest.mark.parametrize("quant", ["fp8_token", "fp8_group", "int8_token"])
+@pytest.mark.parametrize("dtype,code", [(torch.bfloat16, cport.BF16), (torch.float16, cport.F16)])
+def test_c_restatement_propagates_nonfinite_values_like_eager(dtype, code, quant):
+    """NaN and infinities in partials, residual and gamma: the torch ops of the composition propagate NaN (sum, mean,
+    rsqrt, amax, clamp), and the C restatement must make the same rows, scales and codes NaN -- which NaN (sign,
+    payload) is not compared, and int8 codes are not compared where the scaled value is NaN (casting NaN to an
+    integer is undefined in C)."""
+    from helpers import equal_where_not_nan
+    p, r, g = eager.make_inputs(4, 9, 512, dtype, 0.5, seed=91)
+    p[1, 0, 5] = float("nan")
+    p[2, 1, 300] = float("inf")
+    p[0, 2, 40] = float("-inf")
+    r[3, 11] = float("nan")
+    p[3, 4, 7] = float("inf")
+    p[1, 4, 7] = float("-inf")
+    g[100] = float("nan")
+    g[386] = float("inf")
+    want = eager.reduce_rms(p, r, g, 1e-6, quant)
+    c = cport.reduce_rms(code, [_bits16(p[i]) for i in range(4)], _bits16(r), _bits16(g), 1e-6, quant=quant,
+                         sumsq_mode=cport.SUMSQ_TORCH)
+    assert equal_where_not_nan(_from_bits16(c["residual_out"], dtype), want["residual_out"])
+    assert equal_where_not_nan(_from_bits16(c["norm_out"], dtype), want["norm_out"])
+    assert torch.isnan(want["norm_out"].float()).any(dim=1).all()          # gamma's NaN reaches every row
+    assert equal_where_not_nan(torch.from_numpy(c["scale"]).reshape(-1), want["scale"].reshape(-1))
+    got_q = torch.from_numpy(c["q"])
+    if quant == "int8_token":
+        sc = want["scale"].reshape(-1, 1)
+        scaled_nan = torch.isnan(want["norm_out"].float() / torch.where(sc > 0, sc, torch.ones_like(sc)))
+        assert equal_where_not_nan(got_q.view(torch.int8), want["q"], ignore=scaled_nan)
+    else:
+        assert equal_where_not_nan(got_q.view(torch.float8_e4m3fn), want["q"], nan_codes=True)
+
+
 def test_c_restatement_against_eager_over_random_shapes():
     """The two statements of the oracle (torch eager and the integer C restatement in torch's summation order) agree
     bit for bit over a seeded sweep of shapes, element types, numbers of partials and quant modes, including row
