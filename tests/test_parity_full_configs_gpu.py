@@ -12,7 +12,7 @@ import torch
 
 from oracle import eager
 
-from helpers import check_against_oracle, run_hip
+from helpers import bits_equal, check_against_oracle, check_nonfinite, run_hip
 
 pytestmark = pytest.mark.gpu
 
@@ -35,3 +35,25 @@ def test_full_size_configuration_against_oracle(cuda_device, name, tokens):
     if counts_file:
         with open(counts_file, "a") as f:
             f.write(json.dumps(stats) + "\n")
+
+
+@pytest.mark.parametrize("name,tokens", [("c3", None), ("c4", 2048), ("c5", 4096)])
+def test_full_size_configuration_with_nonfinite_values_sprinkled_in(cuda_device, name, tokens):
+    """The configuration's seeded inputs with one element in 20 000 of the partials and of the residual replaced by
+    NaN, +inf or -inf (seeded positions): every output against the oracle with NaN matching NaN, and the rows that
+    stayed finite bit for bit."""
+    parts, residual, gamma, eps, quant = eager.make_config(name, tokens=tokens)
+    g = torch.Generator().manual_seed(977)
+    special = torch.tensor([float("nan"), float("inf"), float("-inf")], dtype=parts.dtype)
+    for t in (parts, residual):
+        flat = t.view(-1)
+        idx = torch.randint(0, flat.numel(), (max(flat.numel() // 20000, 3),), generator=g)
+        flat[idx] = special[torch.randint(0, 3, (idx.numel(),), generator=g)]
+    print("full-size non-finite case", name, tuple(parts.shape), parts.dtype, quant, flush=True)
+    want = eager.reduce_rms(parts, residual, gamma, eps, quant)
+    got = run_hip(parts, residual, gamma, eps, quant)
+    check_nonfinite(got, want, quant)
+    finite_rows = torch.isfinite(want["norm_out"].float()).all(dim=1)
+    assert 0 < int(finite_rows.sum()) < finite_rows.numel()      # both kinds of rows are there
+    assert bits_equal(got["norm_out"][finite_rows], want["norm_out"][finite_rows])
+    assert bits_equal(got["q"][finite_rows], want["q"][finite_rows])

@@ -10,7 +10,7 @@ import torch
 from oracle import eager
 from torch_dist_ext_amd import _capi
 
-from helpers import bits_equal, check_against_oracle, equal_where_not_nan, run_hip, ulp_distance
+from helpers import bits_equal, check_against_oracle, check_nonfinite, run_hip, ulp_distance
 
 pytestmark = pytest.mark.gpu
 
@@ -645,24 +645,6 @@ def test_randomized_launch_geometries(cuda_device):
         _case("geofuzz%d" % k, p, r, g, 1e-6, quant, **kw)
 
 
-def _check_nonfinite(got, want, quant, static_scale=None):
-    """Every output against the oracle's with NaN matching NaN (helpers.equal_where_not_nan); int8 codes are left
-    uncompared where the scaled value is NaN (the oracle's cast of NaN to an integer is undefined in C++)."""
-    assert equal_where_not_nan(got["residual_out"], want["residual_out"]), "residual_out"
-    assert equal_where_not_nan(got["norm_out"], want["norm_out"]), "norm_out"
-    if quant == "none":
-        return
-    if quant != "fp8_static":
-        assert equal_where_not_nan(got["scale"].reshape(-1), want["scale"].reshape(-1)), "scales"
-    if quant == "int8_token":
-        y = want["norm_out"].float()
-        sc = want["scale"].reshape(-1, 1)
-        scaled_nan = torch.isnan(y / torch.where(sc > 0, sc, torch.ones_like(sc)))
-        assert equal_where_not_nan(got["q"], want["q"], ignore=scaled_nan), "int8 codes"
-    else:
-        assert equal_where_not_nan(got["q"], want["q"], nan_codes=True), "fp8 codes"
-
-
 @pytest.mark.parametrize("quant", ["none", "fp8_token", "fp8_group", "int8_token", "fp8_static"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("hidden,vpt", [(256, 0), (2048, 1), (8192, 4), (4096, 2)])
@@ -696,7 +678,7 @@ def test_nonfinite_rows(cuda_device, dtype, quant, hidden, vpt):
         static_scale = 0.0123 if quant == "fp8_static" else None
         want = eager.reduce_rms(p, r, gamma, 1e-5, quant, static_scale=static_scale)
         got = run_hip(p, r, gamma, 1e-5, quant, vecs_per_thread=vpt, static_scale=static_scale or 0.0)
-        _check_nonfinite(got, want, quant)
+        check_nonfinite(got, want, quant)
         # the finite rows with finite gamma are ordinary rows: bit for bit, no NaN anywhere
         if gamma_case == "finite":
             assert not torch.isnan(got["norm_out"][7:].float()).any()
