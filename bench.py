@@ -14,7 +14,8 @@ synchronization that ends them; `roofline.achieved` / `frac` / `kernel_avg_us` a
 stream around the same K launches.  Two states, both in the line: `roofline.cold_kernel_avg_us` is the same
 measurement (W warm-up launches, K timed) taken before the settling phase, `kernel_avg_us` after it.
 `roofline.fit` times the same kernel at three row counts and reports the straight line through them
-(`fixed_us` + bytes / `bulk_GBs`).
+(`fixed_us` + bytes / `bulk_GBs`); `roofline.device_rates_floor` is what the device's own plain read, write and copy
+rates, measured in the same process, make of the launch's bytes.
 Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3] [--no-cpu-baseline] [--settle-ms 20]
@@ -496,6 +497,14 @@ def main():
                                                            stream.cuda_stream), 12, 3)
         rates[name] = moved / (us * 1e-6) / 1e9
     del bufs
+    # What the device's own plain-stream rates make of this launch's bytes: the reads at the read-only rate plus the writes
+    # at the write-only rate, times what the plain copy pays for moving both together, plus one dispatch.  No kernel with
+    # this traffic goes below it on this box; the skeleton (traffic_only_us) is the same thing measured on the real pattern.
+    mixing = (2.0 / rates["copy_GBs"]) / (1.0 / rates["read_only_GBs"] + 1.0 / rates["write_only_GBs"])
+    rates_us = (read_bytes / rates["read_only_GBs"] + max(out_bytes, 0) / rates["write_only_GBs"]) * 1e-3 * mixing + launch_floor_us
+    out["roofline"]["device_rates_floor"] = {
+        "us": rates_us, "frac": bytes_per_launch / (rates_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "copy_mixing_factor": mixing,
+        "what": "reads at device.read_only_GBs + writes at device.write_only_GBs, times the plain copy's cost of moving both together, plus launch_floor_us"}
 
     # The same kernel at three row counts, in blocks of the same rotating buffers (or of larger ones), and the
     # straight line through the three points: time = fixed_us + bytes / bulk_GBs.
