@@ -40,8 +40,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 # They describe the kernels whose sources hash to `sources_sha256`; with any other kernel source the bench line reports
 # traffic as null.
 TRAFFIC = {
-    "sources_sha256": "cb36b78742d24dbc6f8aed6b42621d47f975a3eab81bb4b562febaea200f20fe",
-    "bytes": {"c2": 11696832, "c3": 352648977, "c4": 765464707, "c5": 2181272138},
+    "sources_sha256": "c6d624653c806dc9fcd31ff71092eb38212cd2832b830d6567d9f5a588a69318",
+    "bytes": {"c2": 11696715, "c3": 352660867, "c4": 765466502, "c5": 2181261732},
 }
 
 BENCH_CONFIGS = {

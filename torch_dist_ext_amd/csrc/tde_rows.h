@@ -590,10 +590,25 @@ __global__ void __launch_bounds__(1024 / VPT)
     // own stores, a fresh workgroup does not).
     const int64_t row0 = (int64_t)xcd_chunked_block(blockIdx.x, gridDim.x, (uint32_t)a.xcd_chunk) * a.rows_per_block;
 
-    // The row's loads go out before anything else touches memory.
+    // The row's loads go out before anything else touches memory -- except gamma where it pays to have it first:
+    // with up to four partials of a 2-byte type, several vectors per thread and a per-token scale, the registers are
+    // there to hold gamma through the load phase, and requested ahead of the row (it is served from L2) it is never
+    // waited for behind the row's own traffic.  Measured against requesting it after the accumulate phase, alternating
+    // two builds in one process: 4 x [32768, 5120] fp16 -> int8 per token -1.0 %, 4 x [8192, 7168] bf16 -> fp8 per
+    // token -1.4 %, 2 x [8192, 8192] -0.6 %, 4 x [2048, 7168] -0.7 %; with per-group scales (no second barrier to
+    // cover) +0.9 to +2.7 %, with T-typed output or fp32 rows equal to +0.4 %, so those keep the late request.
+    const rsrc_t gamma_rsrc = row_rsrc(a.gamma, 0, row_bytes);
+    constexpr bool GAMMA_FIRST =
+        VPT > 1 && N != 0 && N <= 4 && E::BYTES == 2 && (Q == TDE_QUANT_FP8_TOKEN || Q == TDE_QUANT_INT8_TOKEN);
+    u32x4 gamma_first[GAMMA_FIRST ? VPT : 1];
+    if constexpr (GAMMA_FIRST) {
+#pragma unroll
+        for (int j = 0; j < VPT; ++j)
+            gamma_first[j] = __builtin_amdgcn_raw_buffer_load_b128(gamma_rsrc, (int)lane_off[j], 0, kAuxDefault);
+        __builtin_amdgcn_sched_barrier(0);
+    }
     RowLoads<NP, VPT> cur;
     issue_loads(cur, row0 + group);
-    const rsrc_t gamma_rsrc = row_rsrc(a.gamma, 0, row_bytes);
     u32x4 gamma_early = u32x4{0, 0, 0, 0};
     if constexpr (VPT == 1) {
         __builtin_amdgcn_sched_barrier(0);
@@ -616,12 +631,13 @@ __global__ void __launch_bounds__(1024 / VPT)
         // ---- reduce, residual add, sum of squares ------------------------------------------------
         const rsrc_t res_out = row_rsrc(a.residual_out, row_byte, bytes);
         u32x4 xraw[VPT];
-        // With several vectors per thread the partials are summed rank by rank as they arrive (the memory system
+        // With four vectors per thread, or one, the partials are summed rank by rank as they arrive (the memory system
         // returns a wavefront's loads in the order it issued them), so that only the last partial's additions are
         // left when the row is complete.  The order of every element's additions is the same either way.  With two
         // vectors per thread the accumulators cost more occupancy than the overlap returns (8 partials, 1024 rows of
-        // 5120: 21.5 us against 20.4), so those variants sum vector by vector.
-        constexpr bool RANK_MAJOR = (N >= 4 && VPT >= 4);
+        // 5120: 21.5 us against 20.4), so those variants sum vector by vector.  With one vector per thread (the
+        // decode-size geometries) waiting rank by rank is worth 0.5-1.5 % up to 512 rows and nothing beyond.
+        constexpr bool RANK_MAJOR = (N >= 4 && (VPT >= 4 || VPT == 1));
         float racc[RANK_MAJOR ? VPT : 1][VEC];
         if constexpr (RANK_MAJOR) {
             __builtin_amdgcn_sched_barrier(0);
@@ -647,6 +663,15 @@ __global__ void __launch_bounds__(1024 / VPT)
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
+        }
+        // From here on the wavefront has its row and only arithmetic, LDS and stores left: with up to four partials
+        // (short load phases, three workgroups sharing the vector units about 60 % of the time) it goes ahead of the
+        // wavefronts that are still summing partials.  4 x [32768, 5120] -0.5 %, 4 x [8192, 7168] -0.2 %; with eight
+        // partials nothing at 2048+ rows and +0.7 % at 512 rows, so those stay at the default priority.
+        if constexpr (N != 0 && N <= 4 && VPT == 4) {
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(1);
+            __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
@@ -680,11 +705,15 @@ __global__ void __launch_bounds__(1024 / VPT)
             sumsq_put<VPT, VEC>(lds_img, j, tpr, group, TDE_T, sq, xraw[j][0]);
         }
         // gamma (shared by all rows, served from L2).  With several vectors per thread it is requested
-        // only now: the registers of the row loads are free again, and the reduction below covers its
-        // latency.  With one vector per thread registers are plentiful and it was requested right
-        // behind the row loads (shortest dependent chain for small, latency-bound inputs).
+        // only now (unless it went out first, see GAMMA_FIRST): the registers of the row loads are free
+        // again, and the reduction below covers its latency.  With one vector per thread registers are
+        // plentiful and it was requested right behind the row loads (shortest dependent chain for small,
+        // latency-bound inputs).
         u32x4 gamma_raw[VPT];
-        if constexpr (VPT > 1) {
+        if constexpr (GAMMA_FIRST) {
+#pragma unroll
+            for (int j = 0; j < VPT; ++j) gamma_raw[j] = gamma_first[j];
+        } else if constexpr (VPT > 1) {
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int j = 0; j < VPT; ++j)
