@@ -29,6 +29,18 @@ def test_library_exports_every_declared_symbol():
     assert _capi.load().tde_abi_version() == _capi.ABI_VERSION == 4
 
 
+def test_library_exports_nothing_but_the_declared_symbols():
+    """Launchers, kernel handles and template instantiations stay inside the library (its link uses an export map),
+    so a second copy of the library in one process runs its own kernels; the dynamic symbol table is read with nm."""
+    import shutil
+    import subprocess
+    if shutil.which("nm") is None:
+        pytest.skip("no nm on this machine")
+    out = subprocess.run(["nm", "-D", "--defined-only", _capi.LIB_PATH], stdout=subprocess.PIPE, text=True, check=True).stdout
+    exported = sorted(line.split()[-1] for line in out.splitlines() if line.strip())
+    assert exported == _declared_functions()
+
+
 def test_struct_layouts_match_header():
     assert ctypes.sizeof(_capi.Problem) == 64
     assert ctypes.sizeof(_capi.Buffers) == (16 + 8) * 8

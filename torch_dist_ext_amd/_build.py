@@ -62,7 +62,10 @@ def build_hip(verbose=False):
 
     with ThreadPoolExecutor(max_workers=6) as pool:
         objs = list(pool.map(compile_one, HIP_SOURCES))
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", HIP_LIB] + objs)
+    # only the C ABI is exported: a second copy of this library in the process (another version, a build under test)
+    # then runs its own launchers and kernels, not the first one's
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,--version-script=" + os.path.join(CSRC, "tde_exports.map"),
+          "-o", HIP_LIB] + objs)
     return HIP_LIB
 
 
