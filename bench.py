@@ -40,8 +40,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 # They describe the kernels whose sources hash to `sources_sha256`; with any other kernel source the bench line reports
 # traffic as null.
 TRAFFIC = {
-    "sources_sha256": "c6d624653c806dc9fcd31ff71092eb38212cd2832b830d6567d9f5a588a69318",
-    "bytes": {"c2": 11696715, "c3": 352660867, "c4": 765466502, "c5": 2181261732},
+    "sources_sha256": "7dd2afe09431dd7fde189054d713f6845c64e8ef7f7a173401b257caa6e420e4",
+    "bytes": {"c2": 11696075, "c3": 352653743, "c4": 765466742, "c5": 2181255870},
 }
 
 BENCH_CONFIGS = {

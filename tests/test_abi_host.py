@@ -321,6 +321,29 @@ def test_plan_workgroups_per_cu(kw, limit, lds):
         assert limit * (lds + 64) <= 160 * 1024 < (limit + 1) * (lds + 64)
 
 
+@pytest.mark.parametrize("kw,limit", [
+    (dict(nranks=8, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_TOKEN), 2),                     # the benchmark's c3
+    (dict(nranks=8, tokens=1024, hidden=8192, dtype=_capi.F16, quant=_capi.QUANT_INT8_TOKEN), 2),  # from 4 workgroups per CU
+    (dict(nranks=8, tokens=4096, hidden=2048, quant=_capi.QUANT_FP8_TOKEN), 2),                     # 4 rows per workgroup: 1024 workgroups
+    (dict(nranks=8, tokens=1023, hidden=8192, quant=_capi.QUANT_FP8_TOKEN), 0),
+    (dict(nranks=8, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_GROUP), 0),
+    (dict(nranks=8, tokens=2048, hidden=8192), 0),                                                   # T-typed output
+    (dict(nranks=8, tokens=2048, hidden=4096, dtype=_capi.F32, quant=_capi.QUANT_FP8_TOKEN), 0),
+    (dict(nranks=4, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_TOKEN), 0),
+    (dict(nranks=8, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_TOKEN, workgroups_per_cu=-1), 0),
+    (dict(nranks=8, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_TOKEN, algo=_capi.ALGO_STAGED), 0),
+])
+def test_plan_picks_the_two_wavefronts_per_simd_kernel(kw, limit):
+    """Eight 2-byte partials, four vectors per thread, per-token scales, 4 to 24 workgroups per CU and no limit asked for:
+    the plan reports two workgroups per CU (the kernel's registers) and leaves the LDS as the geometry needs it."""
+    _needs_256_compute_units()
+    p = _plan(**kw)
+    assert p.workgroups_per_cu == limit
+    unpadded = dict(kw)
+    unpadded["workgroups_per_cu"] = -1
+    assert p.lds_bytes == _plan(**unpadded).lds_bytes
+
+
 @pytest.mark.parametrize("kw", [dict(workgroups_per_cu=9), dict(workgroups_per_cu=-2)])
 def test_plan_rejects_workgroup_limits_out_of_range(kw):
     with pytest.raises(_capi.TdeError) as err:

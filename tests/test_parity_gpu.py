@@ -273,6 +273,26 @@ def test_every_workgroup_limit_agrees(cuda_device, limit, n, hidden, dtype, quan
         assert bits_equal(base[key], other[key]), key
 
 
+@pytest.mark.parametrize("tokens,hidden,dtype,quant", [(1100, 8192, torch.bfloat16, "fp8_token"), (4100, 2048, torch.float16, "int8_token"),
+                                                       (1030, 7168, torch.bfloat16, "int8_token")])
+def test_wide_instantiation_agrees_with_the_plain_one(cuda_device, tokens, hidden, dtype, quant):
+    """Eight 2-byte partials with per-token scales at 4 to 24 workgroups per CU run the row kernel compiled for two
+    wavefronts per SIMD, with gamma requested ahead of the row (the plan reports it as two workgroups per CU);
+    tune_workgroups_per_cu = -1 keeps the plain instantiation.  Same bits from both, and the oracle's."""
+    p, r, g = eager.make_inputs(8, tokens, hidden, dtype, 0.5, seed=191)
+    dcode = _capi.BF16 if dtype == torch.bfloat16 else _capi.F16
+    qcode = _capi.QUANT_FP8_TOKEN if quant == "fp8_token" else _capi.QUANT_INT8_TOKEN
+    auto = _capi.plan(_capi.make_problem(dcode, 8, tokens, hidden, 1e-5, quant=qcode))
+    plain = _capi.plan(_capi.make_problem(dcode, 8, tokens, hidden, 1e-5, quant=qcode, workgroups_per_cu=-1))
+    assert auto.vecs_per_thread == 4 and auto.workgroups_per_cu == 2 and plain.workgroups_per_cu == 0
+    assert auto.lds_bytes == plain.lds_bytes                      # no LDS padding: the registers are the limit
+    wide = run_hip(p, r, g, 1e-5, quant)
+    base = run_hip(p, r, g, 1e-5, quant, workgroups_per_cu=-1)
+    check_against_oracle(wide, eager.reduce_rms(p, r, g, 1e-5, quant), quant, gamma=g, eps=1e-5)
+    for key in base:
+        assert bits_equal(base[key], wide[key]), key
+
+
 def test_long_launch_with_automatic_workgroup_limit(cuda_device):
     """6144 rows of 8 partials: the plan limits the launch to two workgroups per CU (79 KiB of dynamic LDS each).
     Same bits as the unlimited launch, on the device."""

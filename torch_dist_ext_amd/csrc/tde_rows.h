@@ -526,12 +526,15 @@ struct RowLoads {
 //   VPT    16-byte vectors per thread per row (1, 2 or 4)
 //   Q      tde_quant
 //   WN     write the T-typed normed row (always true for Q == NONE)
+//   WIDE   compiled for two wavefronts per SIMD (256 registers) instead of three, with gamma requested ahead of the
+//          row also for eight partials: two workgroups per CU whose gamma never waits.  Launched for eight 2-byte
+//          partials with per-token scales at 4 to 24 workgroups per CU (launch_rows_nv, Geometry::wide)
 // Block layout: rows_per_block row groups of threads_per_row threads; thread t of a row group
 // owns vectors t, t + threads_per_row, ... (coalesced 1 KiB per wavefront per load).
 // ---------------------------------------------------------------------------------------------
-template <class E, int N, int VPT, int Q, bool WN>
+template <class E, int N, int VPT, int Q, bool WN, bool WIDE = false>
 __global__ void __launch_bounds__(1024 / VPT)
-    __attribute__((amdgpu_waves_per_eu(VPT == 1 ? 8 : (VPT == 2 ? 5 : 3)))) row_kernel(const RowArgs a) {
+    __attribute__((amdgpu_waves_per_eu(VPT == 1 ? 8 : (VPT == 2 ? 5 : (WIDE ? 2 : 3))))) row_kernel(const RowArgs a) {
     constexpr int VEC = E::VEC;
     constexpr int NP = (N == 0) ? 1 : N;
     // residual_out is stored together with the row's other output at the end, one write burst per row: against storing
@@ -597,9 +600,14 @@ __global__ void __launch_bounds__(1024 / VPT)
     // two builds in one process: 4 x [32768, 5120] fp16 -> int8 per token -1.0 %, 4 x [8192, 7168] bf16 -> fp8 per
     // token -1.4 %, 2 x [8192, 8192] -0.6 %, 4 x [2048, 7168] -0.7 %; with per-group scales (no second barrier to
     // cover) +0.9 to +2.7 %, with T-typed output or fp32 rows equal to +0.4 %, so those keep the late request.
+    // With eight partials the 16 registers are one too many for three wavefronts per SIMD (169 against 168: spilling
+    // costs 2 us on 8 x [2048, 8192], and gamma ahead of the row for three of the four vectors gains 0.1 us); the WIDE
+    // instantiation takes them and runs two workgroups per CU: 8 x [2048, 8192] bf16 -> fp8 56.8 us against 57.3,
+    // -0.8 % from 1024 to 4096 rows, -1.5 % for rows of 7168, -2.2 % for 4096 rows of 2048, nothing from 6144 rows on
+    // (where the launch is limited to two workgroups per CU anyway) and +0.8 to +1.8 % below 1024 rows.
     const rsrc_t gamma_rsrc = row_rsrc(a.gamma, 0, row_bytes);
-    constexpr bool GAMMA_FIRST =
-        VPT > 1 && N != 0 && N <= 4 && E::BYTES == 2 && (Q == TDE_QUANT_FP8_TOKEN || Q == TDE_QUANT_INT8_TOKEN);
+    constexpr bool GAMMA_FIRST = VPT > 1 && N != 0 && (N <= 4 || WIDE) && E::BYTES == 2 &&
+                                 (Q == TDE_QUANT_FP8_TOKEN || Q == TDE_QUANT_INT8_TOKEN);
     u32x4 gamma_first[GAMMA_FIRST ? VPT : 1];
     if constexpr (GAMMA_FIRST) {
 #pragma unroll
@@ -923,6 +931,7 @@ struct Geometry {
     int block_threads;
     int64_t grid;
     int xcd_chunk;
+    bool wide; // launch the row kernel's WIDE instantiation (eight 2-byte partials, four vectors per thread, per-token scales)
 };
 
 // Per-dtype launchers, defined in tde_rows_<dtype>.hip.
@@ -946,12 +955,22 @@ template <class E, int N, int VPT>
 hipError_t launch_rows_nv(int q, bool wn, const RowArgs &a, const Geometry &g, hipStream_t s) {
     const dim3 grid((unsigned)g.grid), block((unsigned)g.block_threads);
     const size_t lds = (size_t)g.lds_bytes; // sumsq_lds_bytes of this geometry, padded where the launch limits workgroups per CU
-#define TDE_LAUNCH(QM, WNB)                                                         \
-    if (lds > kDefaultMaxDynamicLds) {                                              \
-        const hipError_t e = allow_large_lds<row_kernel<E, N, VPT, QM, WNB>>();     \
-        if (e != hipSuccess) return e;                                              \
-    }                                                                               \
-    hipLaunchKernelGGL((row_kernel<E, N, VPT, QM, WNB>), grid, block, lds, s, a); \
+#define TDE_LAUNCH(QM, WNB)                                                                              \
+    if constexpr (N == 8 && VPT == 4 && E::BYTES == 2 && (QM == TDE_QUANT_FP8_TOKEN || QM == TDE_QUANT_INT8_TOKEN)) { \
+        if (g.wide) {                                                                                    \
+            if (lds > kDefaultMaxDynamicLds) {                                                           \
+                const hipError_t e = allow_large_lds<row_kernel<E, N, VPT, QM, WNB, true>>();            \
+                if (e != hipSuccess) return e;                                                           \
+            }                                                                                            \
+            hipLaunchKernelGGL((row_kernel<E, N, VPT, QM, WNB, true>), grid, block, lds, s, a);        \
+            return hipGetLastError();                                                                    \
+        }                                                                                                \
+    }                                                                                                    \
+    if (lds > kDefaultMaxDynamicLds) {                                                                   \
+        const hipError_t e = allow_large_lds<row_kernel<E, N, VPT, QM, WNB>>();                          \
+        if (e != hipSuccess) return e;                                                                   \
+    }                                                                                                    \
+    hipLaunchKernelGGL((row_kernel<E, N, VPT, QM, WNB>), grid, block, lds, s, a);                      \
     return hipGetLastError();
     switch (q) {
     case TDE_QUANT_NONE: TDE_LAUNCH(TDE_QUANT_NONE, true)
