@@ -40,8 +40,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 # They describe the kernels whose sources hash to `sources_sha256`; with any other kernel source the bench line reports
 # traffic as null.
 TRAFFIC = {
-    "sources_sha256": "7dd2afe09431dd7fde189054d713f6845c64e8ef7f7a173401b257caa6e420e4",
-    "bytes": {"c2": 11696075, "c3": 352653743, "c4": 765466742, "c5": 2181255870},
+    "sources_sha256": "2b24393ed2c0686b5afef913a6d11575d191a6cb4f3f47f1af65b7cce3c2df2b",
+    "bytes": {"c2": 11693808, "c3": 352653802, "c4": 765467669, "c5": 2181243966},
 }
 
 BENCH_CONFIGS = {

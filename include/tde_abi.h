@@ -134,7 +134,7 @@ typedef struct tde_plan_out {
     int32_t workgroups_per_cu; /* limit on resident workgroups per compute unit the launch enforces through its LDS
                                   (0 = none); below a requested tune_workgroups_per_cu where the geometry's own LDS
                                   already admits fewer.  Also 2, without LDS padding, where the plan picks the row
-                                  kernel built for two wavefronts per SIMD (eight 2-byte partials, per-token scales,
+                                  kernel built for two wavefronts per SIMD (eight partials, four vectors per thread,
                                   4 to 24 workgroups per CU, tune_workgroups_per_cu == 0): its registers admit two */
     int32_t lds_bytes;         /* dynamic LDS per workgroup of the row kernel's launch, padding included */
     int64_t algorithmic_bytes; /* (N+1)*T*H*e + H*e + T*H*e + OUT, OUT as documented for the quant mode */

@@ -291,8 +291,9 @@ def test_plan_vectors_per_thread(kw, vpt, threads):
 
 @pytest.mark.parametrize("kw,limit,lds", [
     # fewer than 6144 workgroups, two partials, the staged algorithms and doubles: no limit, LDS = what the reduction needs
-    (dict(nranks=8, tokens=2048, hidden=8192), 0, (256 * 4 * 8 + 1024) * 4),
-    (dict(nranks=8, tokens=6143, hidden=8192), 0, (256 * 4 * 8 + 1024) * 4),
+    # (eight partials at 1024 to 6143 workgroups: the kernel for two wavefronts per SIMD, reported as 2, no LDS padding)
+    (dict(nranks=8, tokens=1023, hidden=8192), 0, (256 * 4 * 8 + 1024) * 4),
+    (dict(nranks=4, tokens=6143, hidden=8192), 0, (256 * 4 * 8 + 1024) * 4),
     (dict(nranks=2, tokens=32768, hidden=8192), 0, (256 * 4 * 8 + 1024) * 4),
     (dict(nranks=8, tokens=32768, hidden=8192, algo=_capi.ALGO_STAGED), 0, (256 * 4 * 8 + 1024) * 4),
     # long launches: about 128 KiB of loads in flight per CU, never fewer than two workgroups or eight wavefronts
@@ -325,17 +326,19 @@ def test_plan_workgroups_per_cu(kw, limit, lds):
     (dict(nranks=8, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_TOKEN), 2),                     # the benchmark's c3
     (dict(nranks=8, tokens=1024, hidden=8192, dtype=_capi.F16, quant=_capi.QUANT_INT8_TOKEN), 2),  # from 4 workgroups per CU
     (dict(nranks=8, tokens=4096, hidden=2048, quant=_capi.QUANT_FP8_TOKEN), 2),                     # 4 rows per workgroup: 1024 workgroups
+    (dict(nranks=8, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_GROUP), 2),
+    (dict(nranks=8, tokens=2048, hidden=8192), 2),                                                   # T-typed output
+    (dict(nranks=8, tokens=2048, hidden=4096, dtype=_capi.F32, quant=_capi.QUANT_FP8_TOKEN), 2),
     (dict(nranks=8, tokens=1023, hidden=8192, quant=_capi.QUANT_FP8_TOKEN), 0),
-    (dict(nranks=8, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_GROUP), 0),
-    (dict(nranks=8, tokens=2048, hidden=8192), 0),                                                   # T-typed output
-    (dict(nranks=8, tokens=2048, hidden=4096, dtype=_capi.F32, quant=_capi.QUANT_FP8_TOKEN), 0),
+    (dict(nranks=8, tokens=2048, hidden=6144, quant=_capi.QUANT_FP8_TOKEN), 0),                     # one vector per thread
+    (dict(nranks=8, tokens=2048, hidden=2048, dtype=_capi.F64), 0),
     (dict(nranks=4, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_TOKEN), 0),
     (dict(nranks=8, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_TOKEN, workgroups_per_cu=-1), 0),
     (dict(nranks=8, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_TOKEN, algo=_capi.ALGO_STAGED), 0),
 ])
 def test_plan_picks_the_two_wavefronts_per_simd_kernel(kw, limit):
-    """Eight 2-byte partials, four vectors per thread, per-token scales, 4 to 24 workgroups per CU and no limit asked for:
-    the plan reports two workgroups per CU (the kernel's registers) and leaves the LDS as the geometry needs it."""
+    """Eight partials, four vectors per thread, 4 to 24 workgroups per CU and no limit asked for: the plan reports two
+    workgroups per CU (the kernel's registers) and leaves the LDS as the geometry needs it."""
     _needs_256_compute_units()
     p = _plan(**kw)
     assert p.workgroups_per_cu == limit

@@ -274,21 +274,26 @@ def test_every_workgroup_limit_agrees(cuda_device, limit, n, hidden, dtype, quan
 
 
 @pytest.mark.parametrize("tokens,hidden,dtype,quant", [(1100, 8192, torch.bfloat16, "fp8_token"), (4100, 2048, torch.float16, "int8_token"),
-                                                       (1030, 7168, torch.bfloat16, "int8_token")])
+                                                       (1030, 7168, torch.bfloat16, "int8_token"), (1100, 8192, torch.float16, "fp8_group"),
+                                                       (1100, 4096, torch.float32, "none"), (1050, 4096, torch.float32, "fp8_token"),
+                                                       (1100, 8192, torch.bfloat16, "none"), (1100, 8192, torch.bfloat16, "fp8_static")])
 def test_wide_instantiation_agrees_with_the_plain_one(cuda_device, tokens, hidden, dtype, quant):
-    """Eight 2-byte partials with per-token scales at 4 to 24 workgroups per CU run the row kernel compiled for two
+    """Eight partials with four vectors per thread at 4 to 24 workgroups per CU run the row kernel compiled for two
     wavefronts per SIMD, with gamma requested ahead of the row (the plan reports it as two workgroups per CU);
     tune_workgroups_per_cu = -1 keeps the plain instantiation.  Same bits from both, and the oracle's."""
     p, r, g = eager.make_inputs(8, tokens, hidden, dtype, 0.5, seed=191)
-    dcode = _capi.BF16 if dtype == torch.bfloat16 else _capi.F16
-    qcode = _capi.QUANT_FP8_TOKEN if quant == "fp8_token" else _capi.QUANT_INT8_TOKEN
-    auto = _capi.plan(_capi.make_problem(dcode, 8, tokens, hidden, 1e-5, quant=qcode))
-    plain = _capi.plan(_capi.make_problem(dcode, 8, tokens, hidden, 1e-5, quant=qcode, workgroups_per_cu=-1))
+    dcode = {torch.bfloat16: _capi.BF16, torch.float16: _capi.F16, torch.float32: _capi.F32}[dtype]
+    qcode = {"none": _capi.QUANT_NONE, "fp8_token": _capi.QUANT_FP8_TOKEN, "fp8_group": _capi.QUANT_FP8_GROUP,
+             "int8_token": _capi.QUANT_INT8_TOKEN, "fp8_static": _capi.QUANT_FP8_STATIC}[quant]
+    static = 0.013 if quant == "fp8_static" else 0.0
+    auto = _capi.plan(_capi.make_problem(dcode, 8, tokens, hidden, 1e-5, quant=qcode, static_scale=static))
+    plain = _capi.plan(_capi.make_problem(dcode, 8, tokens, hidden, 1e-5, quant=qcode, static_scale=static, workgroups_per_cu=-1))
     assert auto.vecs_per_thread == 4 and auto.workgroups_per_cu == 2 and plain.workgroups_per_cu == 0
     assert auto.lds_bytes == plain.lds_bytes                      # no LDS padding: the registers are the limit
-    wide = run_hip(p, r, g, 1e-5, quant)
-    base = run_hip(p, r, g, 1e-5, quant, workgroups_per_cu=-1)
-    check_against_oracle(wide, eager.reduce_rms(p, r, g, 1e-5, quant), quant, gamma=g, eps=1e-5)
+    wide = run_hip(p, r, g, 1e-5, quant, static_scale=static)
+    base = run_hip(p, r, g, 1e-5, quant, static_scale=static, workgroups_per_cu=-1)
+    want = eager.reduce_rms(p, r, g, 1e-5, quant, static_scale=static) if quant == "fp8_static" else eager.reduce_rms(p, r, g, 1e-5, quant)
+    check_against_oracle(wide, want, quant, gamma=g, eps=1e-5)
     for key in base:
         assert bits_equal(base[key], wide[key]), key
 

@@ -191,11 +191,11 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
         // Row groups per XCD chunk of the row mapping (tde_rows.h: xcd_chunked_block); 16 measured best with 8
         // partials, 8 with 4.
         geo->xcd_chunk = p->nranks >= 8 ? 16 : 8;
-        // Eight 2-byte partials, four vectors per thread, per-token scales, no limit asked for or planned, and 4 to 24
-        // workgroups per CU: the row kernel's two-wavefronts-per-SIMD instantiation (tde_rows.h: WIDE) is 0.3-2.2 %
-        // faster there; it is reported as the limit of two workgroups per CU that its registers amount to.
-        geo->wide = p->nranks == 8 && vpt == 4 && eb == 2 && !staged && wgs_per_cu == 0 && p->tune_workgroups_per_cu == 0 &&
-                    (p->quant == TDE_QUANT_FP8_TOKEN || p->quant == TDE_QUANT_INT8_TOKEN) && grid >= 4 * (int64_t)cus;
+        // Eight partials, four vectors per thread, no limit asked for or planned, and 4 to 24 workgroups per CU: the
+        // row kernel's two-wavefronts-per-SIMD instantiation (tde_rows.h: WIDE) is 0.2-2.2 % faster there; it is
+        // reported as the limit of two workgroups per CU that its registers amount to.
+        geo->wide = p->nranks == 8 && vpt == 4 && p->dtype != TDE_F64 && !staged && wgs_per_cu == 0 &&
+                    p->tune_workgroups_per_cu == 0 && grid >= 4 * (int64_t)cus;
         if (geo->wide) geo->wgs_per_cu = 2;
     }
     return TDE_OK;

@@ -527,8 +527,8 @@ struct RowLoads {
 //   Q      tde_quant
 //   WN     write the T-typed normed row (always true for Q == NONE)
 //   WIDE   compiled for two wavefronts per SIMD (256 registers) instead of three, with gamma requested ahead of the
-//          row also for eight partials: two workgroups per CU whose gamma never waits.  Launched for eight 2-byte
-//          partials with per-token scales at 4 to 24 workgroups per CU (launch_rows_nv, Geometry::wide)
+//          row also for eight partials: two workgroups per CU whose gamma never waits.  Launched for eight partials
+//          with four vectors per thread at 4 to 24 workgroups per CU (launch_rows_nv, Geometry::wide)
 // Block layout: rows_per_block row groups of threads_per_row threads; thread t of a row group
 // owns vectors t, t + threads_per_row, ... (coalesced 1 KiB per wavefront per load).
 // ---------------------------------------------------------------------------------------------
@@ -604,10 +604,13 @@ __global__ void __launch_bounds__(1024 / VPT)
     // costs 2 us on 8 x [2048, 8192], and gamma ahead of the row for three of the four vectors gains 0.1 us); the WIDE
     // instantiation takes them and runs two workgroups per CU: 8 x [2048, 8192] bf16 -> fp8 56.8 us against 57.3,
     // -0.8 % from 1024 to 4096 rows, -1.5 % for rows of 7168, -2.2 % for 4096 rows of 2048, nothing from 6144 rows on
-    // (where the launch is limited to two workgroups per CU anyway) and +0.8 to +1.8 % below 1024 rows.
+    // (where the launch is limited to two workgroups per CU anyway) and +0.8 to +1.8 % below 1024 rows.  The other
+    // eight-partial kernels gain less but none loses (per-group scales -1.0 %, T-typed output -0.3 to -0.8 %, fp32 rows
+    // -0.2 to -0.9 %), so WIDE carries gamma ahead of the row for all of them.
     const rsrc_t gamma_rsrc = row_rsrc(a.gamma, 0, row_bytes);
-    constexpr bool GAMMA_FIRST = VPT > 1 && N != 0 && (N <= 4 || WIDE) && E::BYTES == 2 &&
-                                 (Q == TDE_QUANT_FP8_TOKEN || Q == TDE_QUANT_INT8_TOKEN);
+    constexpr bool GAMMA_FIRST =
+        VPT > 1 && N != 0 &&
+        (WIDE || (N <= 4 && E::BYTES == 2 && (Q == TDE_QUANT_FP8_TOKEN || Q == TDE_QUANT_INT8_TOKEN)));
     u32x4 gamma_first[GAMMA_FIRST ? VPT : 1];
     if constexpr (GAMMA_FIRST) {
 #pragma unroll
@@ -931,7 +934,7 @@ struct Geometry {
     int block_threads;
     int64_t grid;
     int xcd_chunk;
-    bool wide; // launch the row kernel's WIDE instantiation (eight 2-byte partials, four vectors per thread, per-token scales)
+    bool wide; // launch the row kernel's WIDE instantiation (eight partials, four vectors per thread)
 };
 
 // Per-dtype launchers, defined in tde_rows_<dtype>.hip.
@@ -956,7 +959,7 @@ hipError_t launch_rows_nv(int q, bool wn, const RowArgs &a, const Geometry &g, h
     const dim3 grid((unsigned)g.grid), block((unsigned)g.block_threads);
     const size_t lds = (size_t)g.lds_bytes; // sumsq_lds_bytes of this geometry, padded where the launch limits workgroups per CU
 #define TDE_LAUNCH(QM, WNB)                                                                              \
-    if constexpr (N == 8 && VPT == 4 && E::BYTES == 2 && (QM == TDE_QUANT_FP8_TOKEN || QM == TDE_QUANT_INT8_TOKEN)) { \
+    if constexpr (N == 8 && VPT == 4) {                                                                  \
         if (g.wide) {                                                                                    \
             if (lds > kDefaultMaxDynamicLds) {                                                           \
                 const hipError_t e = allow_large_lds<row_kernel<E, N, VPT, QM, WNB, true>>();            \
