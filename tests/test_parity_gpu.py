@@ -290,7 +290,7 @@ def test_wide_instantiation_agrees_with_the_plain_one(cuda_device, tokens, hidde
     plain = _capi.plan(_capi.make_problem(dcode, 8, tokens, hidden, 1e-5, quant=qcode, static_scale=static, workgroups_per_cu=-1))
     assert auto.vecs_per_thread == 4 and auto.workgroups_per_cu == 2 and plain.workgroups_per_cu == 0
     assert auto.lds_bytes == plain.lds_bytes                      # no LDS padding: the registers are the limit
-    wide = run_hip(p, r, g, 1e-5, quant, static_scale=static)
+    wide = run_hip(p, r, g, 1e-5, quant, static_scale=static, use_table=(quant == "fp8_token"))   # also through the pointer table
     base = run_hip(p, r, g, 1e-5, quant, static_scale=static, workgroups_per_cu=-1)
     want = eager.reduce_rms(p, r, g, 1e-5, quant, static_scale=static) if quant == "fp8_static" else eager.reduce_rms(p, r, g, 1e-5, quant)
     check_against_oracle(wide, want, quant, gamma=g, eps=1e-5)
