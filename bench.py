@@ -40,8 +40,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
 # They describe the kernels whose sources hash to `sources_sha256`; with any other kernel source the bench line reports
 # traffic as null.
 TRAFFIC = {
-    "sources_sha256": "2b24393ed2c0686b5afef913a6d11575d191a6cb4f3f47f1af65b7cce3c2df2b",
-    "bytes": {"c2": 11693808, "c3": 352653802, "c4": 765467669, "c5": 2181243966},
+    "sources_sha256": "55bb90777cf227977d0f7689232b58b52ca6a471a27da75b4f630d2904ba9706",
+    "bytes": {"c2": 11693631, "c3": 352653693, "c4": 765467842, "c5": 2181249484},
 }
 
 BENCH_CONFIGS = {

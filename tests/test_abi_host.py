@@ -278,8 +278,18 @@ def _needs_256_compute_units():
     (dict(nranks=2, tokens=2048, hidden=8192), 2, 512), (dict(nranks=2, tokens=2049, hidden=8192), 4, 256),
     (dict(nranks=8, tokens=1024, hidden=4096), 4, 128), (dict(nranks=4, tokens=1024, hidden=4096), 1, 512),
     (dict(nranks=8, tokens=2048, hidden=2048), 4, 64), (dict(nranks=8, tokens=2047, hidden=2048), 1, 256),
-    (dict(nranks=4, tokens=32768, hidden=2048), 1, 256),
+    (dict(nranks=4, tokens=32767, hidden=2048), 1, 256), (dict(nranks=4, tokens=32768, hidden=2048), 2, 128),
     (dict(nranks=8, tokens=640, hidden=5120), 2, 320), (dict(nranks=8, tokens=2048, hidden=5120), 1, 640),
+    (dict(nranks=8, tokens=16383, hidden=5120), 1, 640), (dict(nranks=8, tokens=16384, hidden=5120), 2, 320),
+    # long launches of mid-length rows: two vectors per thread
+    (dict(nranks=8, tokens=16383, hidden=4096), 4, 128), (dict(nranks=8, tokens=16384, hidden=4096), 2, 256),
+    (dict(nranks=8, tokens=32767, hidden=2048), 4, 64), (dict(nranks=8, tokens=32768, hidden=2048), 2, 128),
+    (dict(nranks=8, tokens=2047, hidden=6144), 1, 768), (dict(nranks=8, tokens=2048, hidden=6144), 4, 192),
+    (dict(nranks=8, tokens=5632, hidden=6144), 1, 768), (dict(nranks=8, tokens=8192, hidden=6144), 2, 384),
+    (dict(nranks=4, tokens=1024, hidden=6144), 4, 192), (dict(nranks=4, tokens=2048, hidden=6144), 1, 768),
+    (dict(nranks=8, tokens=8191, hidden=3072, quant=_capi.QUANT_FP8_TOKEN), 1, 384), (dict(nranks=8, tokens=8192, hidden=3072, quant=_capi.QUANT_FP8_TOKEN), 4, 128),
+    (dict(nranks=8, tokens=32768, hidden=3072, quant=_capi.QUANT_INT8_TOKEN), 2, 192), (dict(nranks=8, tokens=32768, hidden=3072), 1, 384),
+    (dict(nranks=8, tokens=4096, hidden=1024), 2, 64), (dict(nranks=8, tokens=8192, hidden=1024), 1, 128),
     (dict(nranks=2, tokens=32768, hidden=5120), 2, 320), (dict(nranks=4, tokens=16384, hidden=5120), 4, 192), (dict(nranks=4, tokens=16383, hidden=5120), 2, 320),
 ])
 def test_plan_vectors_per_thread(kw, vpt, threads):
@@ -304,7 +314,7 @@ def test_plan_vectors_per_thread(kw, vpt, threads):
     (dict(nranks=4, tokens=8192, hidden=7168, quant=_capi.QUANT_FP8_TOKEN), 2, 80896),
     (dict(nranks=4, tokens=8191, hidden=7168, quant=_capi.QUANT_FP8_TOKEN), 0, (256 * 4 * 8 + 1024) * 4),   # four partials: from 8192
     (dict(nranks=8, tokens=32768, hidden=1024), 4, 39936),                                   # 2 rows x 18 KiB per workgroup
-    (dict(nranks=4, tokens=32768, hidden=2048), 6, 26112),
+    (dict(nranks=4, tokens=16384, hidden=2048), 6, 26112),
     (dict(nranks=8, tokens=32768, hidden=2048, dtype=_capi.F64), 0, (1024 * 2 + 1024) * 4),   # doubles: 2 per vector, 1024 threads
     # the per-call override
     (dict(nranks=8, tokens=16, hidden=1024, workgroups_per_cu=1), 1, 162816),
@@ -330,7 +340,7 @@ def test_plan_workgroups_per_cu(kw, limit, lds):
     (dict(nranks=8, tokens=2048, hidden=8192), 2),                                                   # T-typed output
     (dict(nranks=8, tokens=2048, hidden=4096, dtype=_capi.F32, quant=_capi.QUANT_FP8_TOKEN), 2),
     (dict(nranks=8, tokens=1023, hidden=8192, quant=_capi.QUANT_FP8_TOKEN), 0),
-    (dict(nranks=8, tokens=2048, hidden=6144, quant=_capi.QUANT_FP8_TOKEN), 0),                     # one vector per thread
+    (dict(nranks=8, tokens=2048, hidden=5120, quant=_capi.QUANT_FP8_TOKEN), 0),                     # one vector per thread
     (dict(nranks=8, tokens=2048, hidden=2048, dtype=_capi.F64), 0),
     (dict(nranks=4, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_TOKEN), 0),
     (dict(nranks=8, tokens=2048, hidden=8192, quant=_capi.QUANT_FP8_TOKEN, workgroups_per_cu=-1), 0),

@@ -107,10 +107,12 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
     int64_t total_bytes = 0; // tokens * hidden * elem must be addressable with 64-bit signed offsets
     if (__builtin_mul_overflow(p->tokens, p->hidden * eb, &total_bytes)) return TDE_ESHAPE;
 
-    // Vectors per thread, from sweeps on MI355X over hidden 1024..8192, 2/4/8 partials and 256..32768 rows (bf16 and
-    // fp16 agree).  Four vectors per thread (small workgroups, many loads in flight per thread, few wavefronts to
-    // synchronize per row, partials summed while the later ones are still arriving) win on long rows and wherever
-    // eight partials meet full wavefronts; elsewhere one vector per thread is as fast or faster.
+    // Vectors per thread, from sweeps on MI355X over hidden 1024..8192 in steps of 1024, 2/4/8 partials, 128..32768 rows
+    // and three output modes (bf16 and fp16 agree); only differences that held on two devices and across the row
+    // counts between the swept powers of two are in here.  Four vectors per thread (small workgroups, many loads in
+    // flight per thread, few wavefronts to synchronize per row, partials summed while the later ones are still
+    // arriving) win on long rows and wherever eight partials meet full wavefronts, two in the longest launches of
+    // mid-length rows; elsewhere one vector per thread is as fast or faster.
     int vpt = 1;
     if (nvec >= 896) {
         // Few rows are latency-bound and the widest row groups have the shortest dependent chain; from 256 rows
@@ -119,9 +121,23 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
         vpt = p->tokens >= 256 ? 4 : (p->tokens >= 128 ? 2 : 1);
         if (p->nranks == 2 && p->tokens >= 256 && p->tokens <= 2048) vpt = 2;
     } else if (nvec == 512 && p->nranks >= 8 && p->tokens >= 1024) {
-        vpt = 4; // 3-4 % over one
+        vpt = p->tokens >= 16384 ? 2 : 4; // four: 3-4 % over one; from 16384 rows two are another 4-7 % ahead
     } else if (nvec == 256 && p->nranks >= 8 && p->tokens >= 2048) {
-        vpt = 4; // 3-6 % over one; with fewer partials or rows one is 3-16 % faster
+        // four: 3-6 % over one (with fewer partials or rows one is 3-16 % faster); from 32768 rows two: another 4-6 %
+        vpt = p->tokens >= 32768 ? 2 : 4;
+    } else if (nvec == 256 && p->nranks == 4 && p->tokens >= 32768) {
+        vpt = 2; // 3-4 % over one
+    } else if (nvec == 768 && p->nranks >= 8 && p->tokens >= 2048) {
+        // rows of 6144 2-byte elements: twelve wavefronts with one vector each lose to three with four vectors
+        // (2048 to 5600 rows: 1.5-2.3 %) and, in long launches, to six with two (3-6 % from 8192 rows)
+        if (p->tokens >= 8192) vpt = 2;
+        else if (p->tokens < 5632) vpt = 4;
+    } else if (nvec == 768 && p->nranks == 4 && p->tokens >= 1024 && p->tokens < 2048) {
+        vpt = 4; // 1-5 %
+    } else if (nvec == 384 && p->nranks >= 8 && p->tokens >= 8192 && p->quant != TDE_QUANT_NONE) {
+        vpt = p->tokens >= 32768 ? 2 : 4; // 4-5 % over one with quantized output; with T-typed output one is 2 % ahead
+    } else if (nvec == 128 && p->nranks >= 8 && p->tokens >= 4096 && p->tokens < 8192) {
+        vpt = 2; // 1-3 % over one
     } else if (nvec == 640) {
         // Ten wavefronts per row leave the compute units unevenly filled: from 640 rows up five wavefronts with two
         // vectors each are 10-21 % faster until there are enough rows to even that out (2048 with eight partials,
@@ -131,6 +147,7 @@ int validate(const tde_problem *p, tde::Geometry *geo) {
         const int64_t even_from = p->nranks >= 8 ? 2048 : (p->nranks == 4 ? 16384 : INT64_MAX);
         if (p->tokens >= 640 && p->tokens < even_from) vpt = 2;
         else if (p->nranks == 4 && p->tokens >= even_from) vpt = 4;
+        else if (p->nranks >= 8 && p->tokens >= 16384) vpt = 2; // eight partials, long launches: 2 % over one
     }
     if (p->tune_vecs_per_thread != 0) {
         if (p->tune_vecs_per_thread != 1 && p->tune_vecs_per_thread != 2 && p->tune_vecs_per_thread != 4) return TDE_EINVAL;
