@@ -298,6 +298,21 @@ def test_wide_instantiation_agrees_with_the_plain_one(cuda_device, tokens, hidde
         assert bits_equal(base[key], wide[key]), key
 
 
+@pytest.mark.parametrize("n,tokens,hidden,dtype,quant,vpt", [
+    (8, 16384, 4096, torch.bfloat16, "fp8_token", 2), (8, 8192, 6144, torch.float16, "int8_token", 2),
+    (8, 2048, 6144, torch.bfloat16, "fp8_group", 4), (4, 32768, 2048, torch.bfloat16, "none", 2),
+    (8, 4100, 1024, torch.float16, "fp8_token", 2)])
+def test_long_launches_of_mid_length_rows(cuda_device, n, tokens, hidden, dtype, quant, vpt):
+    """The geometries the plan picks for long launches of mid-length rows (two or four vectors per thread, several rows per
+    workgroup, a limit on workgroups per CU), whole launches against the oracle."""
+    dcode = _capi.BF16 if dtype == torch.bfloat16 else _capi.F16
+    qcode = {"none": _capi.QUANT_NONE, "fp8_token": _capi.QUANT_FP8_TOKEN, "fp8_group": _capi.QUANT_FP8_GROUP, "int8_token": _capi.QUANT_INT8_TOKEN}[quant]
+    assert _capi.plan(_capi.make_problem(dcode, n, tokens, hidden, 1e-5, quant=qcode)).vecs_per_thread == vpt
+    p, r, g = eager.make_inputs(n, tokens, hidden, dtype, 0.5, seed=233)
+    got = run_hip(p, r, g, 1e-5, quant)
+    check_against_oracle(got, eager.reduce_rms(p, r, g, 1e-5, quant), quant, gamma=g, eps=1e-5)
+
+
 def test_long_launch_with_automatic_workgroup_limit(cuda_device):
     """6144 rows of 8 partials: the plan limits the launch to two workgroups per CU (79 KiB of dynamic LDS each).
     Same bits as the unlimited launch, on the device."""
